@@ -11,6 +11,14 @@
 extern "C" {
 int bw_embed(const int32_t* tokens, const int32_t* feedback, const void* table, int table_is_bf16, float* out,
              int rows, int width, int vocab, void* stream);
+// out[r] = table[token] * scale + pair_table[hash(token before, token)] + pos_table[position], each of the two tables
+// optional.  hash = (before * mul_prev + token * mul_cur) mod buckets; a request's first position takes row ``buckets``.
+// The token before a request's first row of this step is state[slot] (a word per slot), which then takes the request's
+// last token of this step.  seq_rows: [requests, 2] = (first row, rows).  Rows with a negative token or position are zero.
+int bw_embed_sum(const int32_t* tokens, const int32_t* feedback, const int32_t* positions, const int32_t* row_seq,
+                 const int32_t* seq_rows, const int32_t* slots, int32_t* state, const void* table, const void* pair_table,
+                 const void* pos_table, int tables_are_bf16, float scale, int buckets, int mul_prev, int mul_cur,
+                 int max_positions, float* out, int rows, int width, int vocab, void* stream);
 int bw_rmsnorm(const float* x, const void* weight, int weight_is_bf16, void* y, int out_is_bf16, int rows,
                int dim, int ldy, float eps, void* stream);
 int bw_add(float* x, const float* y, long long n, void* stream);
@@ -48,16 +56,20 @@ int bw_gemm_qkv_rope_bf16(const void* x, int ldx, const void* w_qkv, void* q_out
 int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
                      const int32_t* block_table, int table_stride, const float* k_cache, const float* v_cache,
                      float* out, int out_stride, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                     int window, float scale, const float* sink, void* stream);
+                     int window, float scale, const float* sink, int chunk, float softcap, void* stream);
 int bw_attention_f32_tiles(const float* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                            int table_stride, const int32_t* tiles, int num_tiles, int tiled, const float* k_cache,
                            const float* v_cache, float* out, int out_stride, int heads, int kv_heads, int head_dim,
-                           int page_size, int window, float scale, const float* sink, void* stream);
+                           int page_size, int window, float scale, const float* sink, int chunk, float softcap,
+                           void* stream);
 int bw_attention_bf16(const void* q, int q_stride, const int32_t* positions, const int32_t* block_table,
                       int table_stride, const int32_t* tiles, int num_tiles, const void* k_cache,
                       const void* v_cache, int num_pages, void* out, int out_stride, int heads, int kv_heads,
                       int head_dim, int page_size, int window, float scale, int decode, float* scratch,
-                      long long scratch_floats, int32_t* counters, int num_counters, const float* sink, void* stream);
+                      long long scratch_floats, int32_t* counters, int num_counters, const float* sink, int chunk,
+                      float softcap, void* stream);
+// (the three attention entry points above) chunk > 0: a query sees only the keys of its own run of ``chunk`` positions,
+// runs counted from position 0 (not together with a window); softcap > 0: a score s becomes softcap * tanh(s / softcap).
 int bw_attention_decode_scratch(int num_tiles, int heads, int kv_heads, int head_dim, int table_stride,
                                 int page_size, long long* scratch_floats, int* counters);
 int bw_attention_fold_group_tiles(int head_dim);
@@ -105,8 +117,11 @@ int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_off, int k_
 int bw_head_norm_gate(const float* o, int ldi, const float* weight, int wstride, const float* g, int ldg, int gate, void* out,
                       int out_is_bf16, int ldo, const int32_t* positions, int rows, int heads, int vdim, float eps,
                       void* stream);
-// h = act(gate) * up of the stacked 32-bit product [rows, 2*inter]; act 0: SiLU, 1: GELU in its tanh form.
-int bw_glu(const float* gate_up, void* h, int out_is_bf16, int rows, int inter, int act, void* stream);
+// h = act(gate) * up of the stacked 32-bit product [rows, ldg] (gate at column 0, up at column inter); act 0: SiLU,
+// 1: GELU in its tanh form, 2: g = min(gate, limit), u = clamp(up, -limit, limit), h = g sigmoid(alpha g) (u + 1).
+// row_gate (optional): h of row r is multiplied by sigmoid(row_gate[r * ld_row_gate]).
+int bw_glu(const float* gate_up, int ldg, void* h, int out_is_bf16, int rows, int inter, int act, float limit, float alpha,
+           const float* row_gate, int ld_row_gate, void* stream);
 // Attention over a compressed cache shared by all heads (latent_attention.hip).
 int bw_latent_prep(const float* proj, int ldp, int q_off, int dkv_off, const float* norm_w, float eps,
                    const float* cos_table, const float* sin_table, const int32_t* positions, const int32_t* row_seq,
@@ -135,6 +150,15 @@ int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const
                       void* q_out, void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads,
                       int dim, int vdim, int hd, int rot, int page_size, int unit_norm, float eps, int has_kv,
                       int write_cache, void* stream);
+// Queries and keys normed over their whole projection (all heads at once): x / sqrt(mean(x^2) + eps) * w; values as they
+// are or mixed with another layer's values of the same row, v <- (1 - lambda) v + lambda v_first (lambda: one number on
+// the device); the cache write and the queries' copy as bw_pair_rope_unit.  src: [q | k | v] at columns 0, heads*dim,
+// (heads + kv_heads)*dim.  v_keep (optional): receives the row's values as projected (32-bit, [rows, ldk]).
+int bw_whole_norm_kv(const float* src, int lds, const int32_t* positions, const int32_t* row_seq,
+                     const int32_t* block_table, int table_stride, const float* q_w, const float* k_w, float eps,
+                     const float* v_first, int ldf, const float* lambda, float* v_keep, int ldk, void* q_out,
+                     void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads, int dim, int vdim,
+                     int hd, int page_size, int write_cache, void* stream);
 int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
                 int ldo, int rows, int heads, int vdim, void* stream);
 // (y and gates are overwritten: y by its activation, the gates' logits by the recurrence's factor and addend)
@@ -146,18 +170,22 @@ int bw_rglru_scan(float* y, int ldy, const float* y_bias, const float* u, int ld
 int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
                 int rows, int dim, float eps, const int32_t* place, const float* wts, int top, void* stream);
 int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream);
+int bw_scale_rows(float* x, int ld, int rows, int cols, float factor, void* stream);      // x *= factor
 // A feed-forward of routed experts (moe.hip).
-int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
-                 float* wts, void* stream);
+// (weight_scale: the chosen scores are multiplied by it on their way into wts)
+int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, float weight_scale,
+                 int32_t* ids, float* wts, void* stream);
 // route, then plan; one launch for steps of up to 16 rows
-int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
-                      float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream);
+int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, float weight_scale,
+                      int32_t* ids, float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream);
 int bw_moe_max_tiles(int slots, int experts);
 int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
                 int32_t* meta, void* stream);
 int bw_moe_experts(const void* x, int x_is_bf16, int ldx, int x_rows, const void* w, int w_is_bf16, void* out, int ldo,
                    const int32_t* sorted, const int32_t* tiles, const int32_t* meta, int slots, int max_tiles, int top,
                    int K, int N, int gate_up, float limit, float alpha, int round_out, void* stream);
+// (gate_up's activation: limit > 0: g = min(G, limit), u = clamp(U, -limit, limit), h = g sigmoid(alpha g) (u + 1);
+// limit = 0: h = G sigmoid(alpha G) U)
 int bw_moe_tile_rows(int slots);
 int bw_moe_combine(const float* y, int ldy, const int32_t* place, const float* wts, int top, float* out, int ldo,
                    int rows, int width, int accumulate, void* stream);

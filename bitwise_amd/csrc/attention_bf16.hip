@@ -47,6 +47,9 @@ struct AttnBf16Args {
   int heads, kv_heads, page_size, page_shift, num_pages, table_stride, q_stride, out_stride, window, hpt, nsub, num_tiles;
   float scale_log2;           // softmax scale times log2(e)
   const float* sink;          // [heads] or null: a score per head that joins the softmax's denominator and has no value
+  int chunk;                  // > 0: a query sees only the keys of its own run of ``chunk`` positions (runs counted from position 0)
+  float cap_over_scale;       // > 0: scores are soft-capped, s -> cap * tanh(s / cap): cap / scale, and
+  float cap_exp_factor;       //      2 * log2(e) * scale / cap
 };
 
 // What the sink adds to a query's folded sum l, whose terms are taken against the folded maximum m (base-2 domain).
@@ -96,7 +99,8 @@ __device__ __forceinline__ bool group_setup(const AttnBf16Args& a, int first_til
     tc[t].row_c = row0 + (ok ? tok : 0);
     tc[t].head_c = gc.kvh * group + gc.sub * a.hpt + (ok ? hh : 0);
     tc[t].pos_c = ok ? a.positions[tc[t].row_c] : -1;
-    tc[t].lo_c = (a.window > 0 && tc[t].pos_c - a.window + 1 > 0) ? tc[t].pos_c - a.window + 1 : 0;
+    if (a.chunk > 0) tc[t].lo_c = tc[t].pos_c > 0 ? tc[t].pos_c - tc[t].pos_c % a.chunk : 0;
+    else tc[t].lo_c = (a.window > 0 && tc[t].pos_c - a.window + 1 > 0) ? tc[t].pos_c - a.window + 1 : 0;
     kmax = max(kmax, tc[t].pos_c);
     if (tc[t].pos_c >= 0) kmin = min(kmin, tc[t].lo_c);
     // columns without a query do not count: what they compute is finite and never stored
@@ -286,8 +290,22 @@ __device__ __forceinline__ float max_over_lane_groups(float v) {
 // base-2 domain: c = scale * log2(e), m_p = max_j(dot_j) * c, p_j = bf16(exp2(fma(dot_j, c, -m_p))).
 template <int HD>
 __device__ __forceinline__ void softmax_partition(const AttnBf16Args& a, const GroupCtx& gc, const TileCtx<HD>& t,
-                                                  int key0, const f32x4 (&st)[4], float& m_p, u32x4 (&pf)[2]) {
+                                                  int key0, const f32x4 (&dots)[4], float& m_p, u32x4 (&pf)[2]) {
   float mx = -INFINITY;
+  f32x4 st[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) st[u] = dots[u];
+  if (a.cap_over_scale > 0.0f) {
+    // soft cap, still before the scale: (cap / scale) * tanh(d * scale / cap), with tanh(x) = 1 - 2 / (1 + e^(2x)),
+    // which ends at -1 and 1 for arguments far out without an overflow that matters
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e2 = __builtin_amdgcn_exp2f(st[u][i] * a.cap_exp_factor);
+        st[u][i] = a.cap_over_scale * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e2));
+      }
+  }
   if (key0 >= t.all_lo && key0 + ATT_PART - 1 <= t.all_hi) {
     // every key of the partition is visible to every column: the same statements without the masks
 #pragma unroll
@@ -897,7 +915,7 @@ __global__ __launch_bounds__(64 * W) __attribute__((amdgpu_waves_per_eu(2))) voi
   // Without a window and with the implicit tile list the first partition is partition 0 of sequence blockIdx.x
   // whatever the position says: its pages are asked for beside the position, not after it (the table index is
   // clamped into the row and the pages into the pool, so a sequence shorter than that costs a wasted load).
-  const bool early = a.window == 0 && a.tiles == nullptr;
+  const bool early = a.window == 0 && a.chunk == 0 && a.tiles == nullptr;
   PartPages pg_first;
   if (early) {
     gc.r = threadIdx.x & 15;
@@ -1125,9 +1143,10 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
                                  const void* v_cache, int num_pages, void* out, int out_stride, int heads,
                                  int kv_heads, int head_dim, int page_size, int window, float scale, int decode,
                                  float* scratch, long long scratch_floats, int32_t* counters, int num_counters,
-                                 const float* sink, void* stream) {
+                                 const float* sink, int chunk, float softcap, void* stream) {
   if (num_tiles <= 0) return 0;
   if (num_pages <= 0) return -2;
+  if (chunk < 0 || (chunk > 0 && window > 0) || softcap < 0.0f) return -2;
   if (kv_heads <= 0 || heads % kv_heads) return -2;
   if (page_size < 4 || (page_size & (page_size - 1)) || page_size > ATT_PART) return -5;  // 4-key loads stay inside a page
   if ((q_stride % 8) || (out_stride % 4)) return -3;
@@ -1146,6 +1165,9 @@ extern "C" int bw_attention_bf16(const void* q, int q_stride, const int32_t* pos
   a.sink = sink;
   if (!(scale > 0.0f)) return -2;                // the maximum is taken before the scaling
   a.scale_log2 = scale * 1.44269504088896340736f;
+  a.chunk = chunk;
+  a.cap_over_scale = softcap > 0.0f ? softcap / scale : 0.0f;
+  a.cap_exp_factor = softcap > 0.0f ? 2.0f * 1.44269504088896340736f * scale / softcap : 0.0f;
   if (kv_heads * a.nsub > 65535) return -2;
   if ((long long)kv_heads * page_size * head_dim * 2 >= (1ll << 31)) return -2;    // a page's bytes as a 32-bit factor
   hipStream_t s = (hipStream_t)stream;

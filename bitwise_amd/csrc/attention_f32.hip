@@ -26,7 +26,22 @@ struct AttnF32Args {
   int page_shift;            // log2 of the page size, or -1 if it is no power of two
   const int32_t* tiles;      // [tiles][4] = row0, tokens, seq, 0 (consecutive rows of one sequence); null: a row a workgroup
   const float* sink;         // [heads] or null: a score per head that joins the softmax's denominator and has no value
+  int chunk;                 // > 0: a query sees only the keys of its own run of ``chunk`` positions (runs counted from position 0)
+  float softcap;             // > 0: a score s becomes softcap * tanh(s / softcap) before the softmax
 };
+
+// The first key a query at ``pos`` sees: the start of its chunk, the window's first position, or 0.  It never
+// decreases with the position.
+__device__ __forceinline__ int first_key(const AttnF32Args& a, int pos) {
+  if (a.chunk > 0) return pos > 0 ? pos - pos % a.chunk : 0;
+  return first_key(a, pos);
+}
+
+// A score from the dot product of a query and a key.
+__device__ __forceinline__ float att_score(const AttnF32Args& a, float dot) {
+  const float s = dot * a.scale;
+  return a.softcap > 0.0f ? a.softcap * tanhf(s / a.softcap) : s;
+}
 
 // What the sink adds to a query's sum of exponentials taken against the maximum mx of its keys' scores (the keys'
 // terms stay as they are; a sink far above every key gives a huge term and an output of zero).
@@ -153,7 +168,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
   if (table_fits)
     for (int i = tid; i < pages; i += T) table_lds[i] = table[i];
   __syncthreads();
-  const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+  const int lo = first_key(a, pos);
   const size_t head_off = (size_t)kvh * a.page_size * HD;
   const size_t page_stride = (size_t)a.kv_heads * a.page_size * HD;
   // element offset of key j (clamped to the last key: loads past it stay inside the sequence and go unused)
@@ -198,7 +213,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
 #pragma unroll
         for (int c = 0; c < NC; ++c) chain = fmaf(qr[c], kr[d][c], chain);
         fetch_key(kr[d], j + DEPTH * G);                           // (past the last key: the last key again, unused)
-        const float sc = row16_sum(chain) * a.scale;
+        const float sc = att_score(a, row16_sum(chain));
         if (j <= pos) {
           if constexpr (KEEP) {
             if (t == 0) scores[j - lo] = sc;
@@ -240,7 +255,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_kernel(AttnF32Arg
   auto park = [&](int j0, int buf) {                       // ``krow`` holds key j0 + et; afterwards key j0 + KC + et
     if (KEEP || et < 0) return;
     const int j = j0 + et;
-    const float e = bw_expf(dot_canonical<HD>(q_lds, krow) * a.scale - mx);
+    const float e = bw_expf(att_score(a, dot_canonical<HD>(q_lds, krow)) - mx);
     load_row<HD>(krow, a.k_cache + offset_of(j + KC));
     e_lds[buf][et] = j <= pos ? e : 0.0f;
   };
@@ -456,11 +471,11 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
   const bool active = qi < ntok;
   const int my_row = row0 + (active ? qi : 0);
   const int pos_q = active ? a.positions[my_row] : -1;              // a padding row: nothing to do either
-  const int lo_q = (a.window > 0 && pos_q - a.window + 1 > 0) ? pos_q - a.window + 1 : 0;
+  const int lo_q = first_key(a, pos_q);
   // the tile's keys: from the first key any query sees to the last one (rows are in position order)
   const int pos_first = a.positions[row0], pos_last = a.positions[row0 + ntok - 1];
   if (pos_last < 0) return;
-  const int lo_min = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
+  const int lo_min = first_key(a, pos_first);
   const int kvh = h / (a.heads / a.kv_heads);
   const size_t head_off = (size_t)kvh * a.page_size * HD;
   const size_t page_stride = (size_t)a.kv_heads * a.page_size * HD;
@@ -510,7 +525,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
 #pragma unroll
     for (int u = 0; u < CH / 16; ++u) {
       const int key = c0 + kl + 16 * u;
-      if (key >= lo_q && key <= pos_q) mx = fmaxf(mx, dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR) * a.scale);
+      if (key >= lo_q && key <= pos_q) mx = fmaxf(mx, att_score(a, dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR)));
     }
   }
   mx = row16_max(mx);
@@ -529,7 +544,7 @@ __global__ __launch_bounds__(ATT32_THREADS) void attention_f32_tile_kernel(AttnF
     for (int u = 0; u < CH / 16; ++u) {
       const int key = c0 + kl + 16 * u;
       float e = 0.0f;
-      if (key >= lo_q && key <= pos_q) e = bw_expf(dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR) * a.scale - mx);
+      if (key >= lo_q && key <= pos_q) e = bw_expf(att_score(a, dot_canonical_lds<HD>(q, k_lds + (kl + 16 * u) * KSTR)) - mx);
       e_lds[qi * CH + kl + 16 * u] = e;
     }
     __syncthreads();
@@ -678,11 +693,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const bool active = col < ntok;
   const int my_row = row0 + (active ? col : ntok - 1);
   const int pos_q = active ? a.positions[my_row] : -1;
-  const int lo_q = (a.window > 0 && pos_q - a.window + 1 > 0) ? pos_q - a.window + 1 : 0;
+  const int lo_q = first_key(a, pos_q);
   const int pos_first = a.positions[row0], pos_last = a.positions[row0 + ntok - 1];
   if (pos_last < 0) return;
-  const int lo_min = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
-  const int lo_last = (a.window > 0 && pos_last - a.window + 1 > 0) ? pos_last - a.window + 1 : 0;   // the last row's first key
+  const int lo_min = first_key(a, pos_first);
+  const int lo_last = first_key(a, pos_last);   // the last row's first key
   const int kvh = h / (a.heads / a.kv_heads);
   const float* kc = a.k_cache + (size_t)kvh * a.page_size * HD;     // this head's rows of page 0
   const float* vc = a.v_cache + (size_t)kvh * a.page_size * HD;
@@ -757,11 +772,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if ((KB) + 64 <= pos_last) fetch_keys((KB) + 64, page, slot, KR);                    \
       __builtin_amdgcn_sched_barrier(0);                                                   \
       if ((KB) + 31 <= pos_first && (KB) >= lo_last) {       /* every query of the tile sees every key of the block */ \
-        _Pragma("unroll") for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r] * a.scale);     \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) mx = fmaxf(mx, att_score(a, s[r])); \
       } else {                                                                             \
         _Pragma("unroll") for (int r = 0; r < 16; ++r) {                                   \
           const int key = (KB) + 8 * (r >> 2) + key_of_reg + (r & 3);                      \
-          const float t = fmaxf(mx, s[r] * a.scale);                                       \
+          const float t = fmaxf(mx, att_score(a, s[r]));                                   \
           mx = (key >= lo_q && key <= pos_q) ? t : mx;                                     \
         }                                                                                  \
       }                                                                                    \
@@ -838,10 +853,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (!((KB) + 31 <= pos_first && (KB) >= lo_last)) {                                                               \
         _Pragma("unroll") for (int r = 0; r < 16; ++r) {                                                                \
           const int key = (KB) + 8 * (r >> 2) + key_of_reg + (r & 3);                                                   \
-          e[r] = (key >= lo_q && key <= pos_q) ? e[r] * a.scale - mx : -200.0f;                                         \
+          e[r] = (key >= lo_q && key <= pos_q) ? att_score(a, e[r]) - mx : -200.0f;                                     \
         }                                                                                                               \
       } else {                                                                                                          \
-        _Pragma("unroll") for (int r = 0; r < 16; ++r) e[r] = e[r] * a.scale - mx;                                      \
+        _Pragma("unroll") for (int r = 0; r < 16; ++r) e[r] = att_score(a, e[r]) - mx;                                  \
       }                                                                                                                 \
       __builtin_amdgcn_sched_barrier(0);                                                                                \
       _Pragma("unroll") for (int g2 = 0; g2 < 4; ++g2) {                                                                \
@@ -916,6 +931,7 @@ static void launch_attention_f32(const AttnF32Args& a, dim3 grid, hipStream_t s)
   // the most keys a query of this launch can see: what a row of the block table covers, or the window
   long long capacity = (long long)a.table_stride * a.page_size;
   if (a.window > 0 && a.window < capacity) capacity = a.window;
+  if (a.chunk > 0 && a.chunk < capacity) capacity = a.chunk;
   const long long keep_bytes = Att32Shape<HD>::LDS_BYTES + ((capacity + 3) & ~3ll) * (long long)sizeof(float);
   if (keep_bytes <= ATT32_KEEP_LDS && a.table_stride <= ATT32_TABLE && a.page_shift >= 0)   // (and the table's row fits the kernel's copy of it)
     hipLaunchKernelGGL((attention_f32_kernel<HD, true>), grid, dim3(ATT32_THREADS), (size_t)keep_bytes, s, a);
@@ -947,11 +963,13 @@ static int attention_f32_dispatch(const AttnF32Args& a, int items, int tiled, hi
 extern "C" int bw_attention_f32(const float* q, int q_stride, const int32_t* positions, const int32_t* row_seq,
                                 const int32_t* block_table, int table_stride, const float* k_cache,
                                 const float* v_cache, float* out, int out_stride, int rows, int heads,
-                                int kv_heads, int head_dim, int page_size, int window, float scale, const float* sink, void* stream) {
+                                int kv_heads, int head_dim, int page_size, int window, float scale, const float* sink, int chunk,
+                                float softcap, void* stream) {
   if (rows <= 0) return 0;
+  if (chunk < 0 || (chunk > 0 && window > 0) || softcap < 0.0f) return -2;
   AttnF32Args a{q, positions, row_seq, block_table, k_cache, v_cache, out, rows, heads, kv_heads, head_dim,
                 page_size, table_stride, q_stride, out_stride, window, scale,
-                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, nullptr, sink};
+                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, nullptr, sink, chunk, softcap};
   return attention_f32_dispatch(a, rows, 0, (hipStream_t)stream);
 }
 
@@ -963,11 +981,12 @@ extern "C" int bw_attention_f32_tiles(const float* q, int q_stride, const int32_
                                       int table_stride, const int32_t* tiles, int num_tiles, int tiled,
                                       const float* k_cache, const float* v_cache, float* out, int out_stride, int heads,
                                       int kv_heads, int head_dim, int page_size, int window, float scale, const float* sink,
-                                      void* stream) {
+                                      int chunk, float softcap, void* stream) {
   if (num_tiles <= 0) return 0;
+  if (chunk < 0 || (chunk > 0 && window > 0) || softcap < 0.0f) return -2;
   if (tiles == nullptr) return -2;
   AttnF32Args a{q, positions, nullptr, block_table, k_cache, v_cache, out, 0, heads, kv_heads, head_dim,
                 page_size, table_stride, q_stride, out_stride, window, scale,
-                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, tiles, sink};
+                (page_size & (page_size - 1)) == 0 ? __builtin_ctz((unsigned)page_size) : -1, tiles, sink, chunk, softcap};
   return attention_f32_dispatch(a, num_tiles, tiled, (hipStream_t)stream);
 }

@@ -42,6 +42,92 @@ extern "C" int bw_embed(const int32_t* tokens, const int32_t* feedback, const vo
   return BW_LAUNCH_CHECK();
 }
 
+// The sum of up to three tables' rows: the token's row times a scale, a row of a table of token pairs chosen by a hash of
+// (token before, token), and the position's row.  A workgroup a row.  The token before a request's first row of the
+// step is the word the request's slot holds; the workgroup of that first row reads it and then leaves the request's
+// last token of the step there, so no other workgroup touches the word.
+template <typename TableT>
+__global__ void embed_sum_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ feedback,
+                                 const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
+                                 const int32_t* __restrict__ seq_rows, const int32_t* __restrict__ slots,
+                                 int32_t* __restrict__ state, const TableT* __restrict__ table,
+                                 const TableT* __restrict__ pair_table, const TableT* __restrict__ pos_table, float scale,
+                                 int buckets, int mul_prev, int mul_cur, int max_positions, float* __restrict__ out,
+                                 int width, int vocab) {
+  const int row = blockIdx.x;
+  auto token_of = [&](int r) {
+    int t = tokens[r];
+    if (t == BW_TOKEN_FROM_FEEDBACK && feedback != nullptr) t = feedback[r];
+    return t;
+  };
+  const int tok = token_of(row);
+  const int pos = positions[row];
+  float* o = out + (size_t)row * width;
+  if (tok < 0 || tok >= vocab || pos < 0 || pos >= max_positions) {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = 0.0f;
+    return;
+  }
+  __shared__ int pair_row;
+  if (threadIdx.x == 0) {
+    int pr = buckets;                                   // a request's first token: the row behind the hashed ones
+    if (pair_table != nullptr) {
+      const int seq = row_seq[row];
+      const int first = seq_rows[2 * seq], n = seq_rows[2 * seq + 1], slot = slots[seq];
+      int before = -1;
+      if (row > first) before = token_of(row - 1);
+      else if (slot >= 0) before = state[slot];
+      if (pos > 0 && before >= 0)
+        pr = (int)(((long long)before * mul_prev + (long long)tok * mul_cur) % buckets);
+      if (row == first && slot >= 0) {
+        const int last = token_of(first + n - 1);
+        if (last >= 0) state[slot] = last;
+      }
+    }
+    pair_row = pr;
+  }
+  __syncthreads();
+  const TableT* e = table + (size_t)tok * width;
+  const TableT* b = pair_table != nullptr ? pair_table + (size_t)pair_row * width : nullptr;
+  const TableT* p = pos_table != nullptr ? pos_table + (size_t)pos * width : nullptr;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v, vb = 0.0f, vp = 0.0f;
+    if constexpr (sizeof(TableT) == 2) {
+      v = bf16_to_f32(e[i]);
+      if (b != nullptr) vb = bf16_to_f32(b[i]);
+      if (p != nullptr) vp = bf16_to_f32(p[i]);
+    } else {
+      v = e[i];
+      if (b != nullptr) vb = b[i];
+      if (p != nullptr) vp = p[i];
+    }
+    v = v * scale;
+    if (b != nullptr) v = v + vb;
+    if (p != nullptr) v = v + vp;
+    o[i] = v;
+  }
+}
+
+extern "C" int bw_embed_sum(const int32_t* tokens, const int32_t* feedback, const int32_t* positions, const int32_t* row_seq,
+                            const int32_t* seq_rows, const int32_t* slots, int32_t* state, const void* table,
+                            const void* pair_table, const void* pos_table, int tables_are_bf16, float scale, int buckets,
+                            int mul_prev, int mul_cur, int max_positions, float* out, int rows, int width, int vocab,
+                            void* stream) {
+  if (rows <= 0) return 0;
+  if (positions == nullptr || table == nullptr) return -2;
+  if (pair_table != nullptr && (buckets <= 0 || row_seq == nullptr || seq_rows == nullptr || slots == nullptr || state == nullptr))
+    return -2;
+  hipStream_t s = (hipStream_t)stream;
+  if (tables_are_bf16)
+    hipLaunchKernelGGL(embed_sum_kernel<bf16_t>, dim3(rows), dim3(256), 0, s, tokens, feedback, positions, row_seq, seq_rows, slots,
+                       state, (const bf16_t*)table, (const bf16_t*)pair_table, (const bf16_t*)pos_table, scale, buckets, mul_prev,
+                       mul_cur, max_positions, out, width, vocab);
+  else
+    hipLaunchKernelGGL(embed_sum_kernel<float>, dim3(rows), dim3(256), 0, s, tokens, feedback, positions, row_seq, seq_rows, slots,
+                       state, (const float*)table, (const float*)pair_table, (const float*)pos_table, scale, buckets, mul_prev,
+                       mul_cur, max_positions, out, width, vocab);
+  return BW_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------------- RMSNorm, 32-bit
 
 // 16 lanes per row: lane j runs the fused multiply-add chain over i = j, j+16, ... and the

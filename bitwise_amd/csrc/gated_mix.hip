@@ -223,6 +223,96 @@ extern "C" int bw_pair_rope_unit(const float* src, int lds, const int32_t* posit
   return BW_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------------------ norm over whole projections, value mixing
+
+struct WholeNormArgs {
+  const float* src;
+  const int32_t* positions;
+  const int32_t* row_seq;
+  const int32_t* block_table;
+  const float* q_w;
+  const float* k_w;
+  const float* v_first;
+  const float* lambda;
+  float* v_keep;
+  void* q_out;
+  void* k_cache;
+  void* v_cache;
+  int lds, ldf, ldk, heads, kv_heads, dim, vdim, hd, page_size, table_stride, write_cache;
+  float eps;
+};
+
+// The workgroup's sum of one number a thread: the waves' sums (xor butterflies) added in wave order.
+__device__ __forceinline__ float workgroup_sum_256(float v, float* lds4) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float t = ((lds4[0] + lds4[1]) + lds4[2]) + lds4[3];
+  __syncthreads();
+  return t;
+}
+
+// A workgroup a row.
+template <typename T>
+__global__ __launch_bounds__(256) void whole_norm_kv_kernel(WholeNormArgs a) {
+  __shared__ float red[4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const int pos = a.positions[row];
+  if (pos < 0) return;
+  const int qn = a.heads * a.dim, kn = a.kv_heads * a.dim, vn = a.kv_heads * a.vdim;
+  const float* q = a.src + (size_t)row * a.lds;
+  const float* k = q + qn;
+  const float* v = k + kn;
+  float acc = 0.0f;
+  for (int i = tid; i < qn; i += 256) acc = fmaf(q[i], q[i], acc);
+  const float inv_q = 1.0f / sqrtf(workgroup_sum_256(acc, red) / (float)qn + a.eps);
+  T* qo = reinterpret_cast<T*>(a.q_out) + (size_t)row * a.heads * a.hd;
+  for (int i = tid; i < a.heads * a.hd; i += 256) {
+    const int h = i / a.hd, d = i % a.hd;
+    gm_store(qo + i, d < a.dim ? (q[h * a.dim + d] * inv_q) * a.q_w[h * a.dim + d] : 0.0f);
+  }
+  if (!a.write_cache) return;
+  acc = 0.0f;
+  for (int i = tid; i < kn; i += 256) acc = fmaf(k[i], k[i], acc);
+  const float inv_k = 1.0f / sqrtf(workgroup_sum_256(acc, red) / (float)kn + a.eps);
+  const int page = a.block_table[(size_t)a.row_seq[row] * a.table_stride + pos / a.page_size];
+  const int slot = pos % a.page_size;
+  T* kc = reinterpret_cast<T*>(a.k_cache);
+  T* vc = reinterpret_cast<T*>(a.v_cache);
+  const float lam = a.v_first != nullptr ? a.lambda[0] : 0.0f;
+  for (int i = tid; i < a.kv_heads * a.hd; i += 256) {
+    const int h = i / a.hd, d = i % a.hd;
+    gm_store(kc + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * a.hd + d,
+             d < a.dim ? (k[h * a.dim + d] * inv_k) * a.k_w[h * a.dim + d] : 0.0f);
+    float val = 0.0f;
+    if (d < a.vdim) {
+      val = v[h * a.vdim + d];
+      if (a.v_keep != nullptr) a.v_keep[(size_t)row * a.ldk + h * a.vdim + d] = val;
+      if (a.v_first != nullptr) val = (1.0f - lam) * val + lam * a.v_first[(size_t)row * a.ldf + h * a.vdim + d];
+    }
+    if constexpr (sizeof(T) == 2) gm_store(vc + (((size_t)page * a.kv_heads + h) * a.hd + d) * a.page_size + slot, val);   // [kv head][element][slot]
+    else gm_store(vc + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * a.hd + d, val);
+  }
+}
+
+extern "C" int bw_whole_norm_kv(const float* src, int lds, const int32_t* positions, const int32_t* row_seq,
+                                const int32_t* block_table, int table_stride, const float* q_w, const float* k_w, float eps,
+                                const float* v_first, int ldf, const float* lambda, float* v_keep, int ldk, void* q_out,
+                                void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads, int dim, int vdim,
+                                int hd, int page_size, int write_cache, void* stream) {
+  if (rows <= 0) return 0;
+  if (heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || dim > hd || vdim > hd || page_size <= 0) return -2;
+  if (lds < heads * dim + (write_cache ? kv_heads * (dim + vdim) : 0)) return -2;
+  if (v_first != nullptr && (lambda == nullptr || ldf < kv_heads * vdim)) return -2;
+  if (v_keep != nullptr && ldk < kv_heads * vdim) return -2;
+  if (v_keep != nullptr && v_keep == v_first) return -2;
+  WholeNormArgs a{src, positions, row_seq, block_table, q_w, k_w, v_first, lambda, v_keep, q_out, k_cache, v_cache, lds, ldf, ldk,
+                  heads, kv_heads, dim, vdim, hd, page_size, table_stride, write_cache, eps};
+  if (is_bf16) hipLaunchKernelGGL(whole_norm_kv_kernel<bf16_t>, dim3(rows), dim3(256), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(whole_norm_kv_kernel<float>, dim3(rows), dim3(256), 0, (hipStream_t)stream, a);
+  return BW_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------------------ output gate
 
 template <typename TI, typename TO>
@@ -431,6 +521,19 @@ __global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ x, int
   if (e >= cols) return;
   float* p = x + (size_t)blockIdx.y * ld + e;
   *p = cap * tanhf(*p / cap);
+}
+
+__global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ x, int ld, int rows, int cols, float factor) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= cols) return;
+  for (int r = blockIdx.y; r < rows; r += gridDim.y) x[(size_t)r * ld + e] *= factor;
+}
+
+extern "C" int bw_scale_rows(float* x, int ld, int rows, int cols, float factor, void* stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  hipLaunchKernelGGL(scale_rows_kernel, dim3((cols + 255) / 256, rows < 65535 ? rows : 65535), dim3(256), 0, (hipStream_t)stream, x, ld,
+                     rows, cols, factor);
+  return BW_LAUNCH_CHECK();
 }
 
 extern "C" int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream) {

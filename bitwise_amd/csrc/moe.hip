@@ -41,7 +41,7 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 
 // A wave a row.  LDS of the wave: scores [E], group scores [count], allowed [count].
 __device__ __forceinline__ void route_row(const float* __restrict__ logits, int ld, int row, int E, int top, int count, int keep,
-                                          int32_t* __restrict__ ids, float* __restrict__ wts, float* s, int lane) {
+                                          float weight_scale, int32_t* __restrict__ ids, float* __restrict__ wts, float* s, int lane) {
   float* gs = s + E;
   float* allowed = gs + count;
   const float* z = logits + (size_t)row * ld;
@@ -86,7 +86,7 @@ __device__ __forceinline__ void route_row(const float* __restrict__ logits, int 
     wave_argmax(v, i);
     if (lane == 0) {
       ids[(size_t)row * top + it] = i;
-      wts[(size_t)row * top + it] = v;
+      wts[(size_t)row * top + it] = v * weight_scale;
       s[i] = -3.0f;
     }
     __builtin_amdgcn_wave_barrier();
@@ -94,23 +94,24 @@ __device__ __forceinline__ void route_row(const float* __restrict__ logits, int 
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
-                                                        int keep, int32_t* __restrict__ ids, float* __restrict__ wts) {
+                                                        int keep, float weight_scale, int32_t* __restrict__ ids,
+                                                        float* __restrict__ wts) {
   extern __shared__ float route_lds[];
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + wave;
   if (row >= rows) return;
-  route_row(logits, ld, row, E, top, count, keep, ids, wts, route_lds + (size_t)wave * (E + 2 * count), lane);
+  route_row(logits, ld, row, E, top, count, keep, weight_scale, ids, wts, route_lds + (size_t)wave * (E + 2 * count), lane);
 }
 
-extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
-                            float* wts, void* stream) {
+extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, float weight_scale,
+                            int32_t* ids, float* wts, void* stream) {
   if (rows <= 0) return 0;
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || groups < 1 || experts % groups || keep < 1 || keep > groups ||
       top > keep * (experts / groups))
     return -2;
   const size_t bytes = (size_t)4 * (experts + 2 * groups) * sizeof(float);
   hipLaunchKernelGGL(moe_route_kernel, dim3((rows + 3) / 4), dim3(256), bytes, (hipStream_t)stream, logits, ld, rows, experts, top,
-                     groups, keep, ids, wts);
+                     groups, keep, weight_scale, ids, wts);
   return BW_LAUNCH_CHECK();
 }
 
@@ -193,12 +194,12 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
 
 // Steps of up to 16 rows: route (a wave a row) and plan in one launch of one workgroup.
 __global__ __launch_bounds__(1024) void moe_route_plan_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
-                                                              int keep, int32_t* __restrict__ ids, float* __restrict__ wts, int segs,
+                                                              int keep, float weight_scale, int32_t* __restrict__ ids, float* __restrict__ wts, int segs,
                                                               int tm, int32_t* __restrict__ sorted, int32_t* __restrict__ place,
                                                               int32_t* __restrict__ tiles, int32_t* __restrict__ meta) {
   extern __shared__ float both_lds[];   // the waves' routing tables, then the plan's slots
   const int wave = wave_index(), lane = threadIdx.x & 63;
-  if (wave < rows) route_row(logits, ld, wave, E, top, count, keep, ids, wts, both_lds + (size_t)wave * (E + 2 * count), lane);
+  if (wave < rows) route_row(logits, ld, wave, E, top, count, keep, weight_scale, ids, wts, both_lds + (size_t)wave * (E + 2 * count), lane);
   __syncthreads();                      // (the rows' choices, written to memory by their waves, are visible to the workgroup)
   plan_body(ids, rows * top, E, segs, tm, 1, reinterpret_cast<int*>(both_lds + (size_t)rows * (E + 2 * count)), sorted, place, tiles, meta);
 }
@@ -223,25 +224,26 @@ extern "C" int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* 
   return BW_LAUNCH_CHECK();
 }
 
-extern "C" int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, int32_t* ids,
-                                 float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream) {
+extern "C" int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep,
+                                 float weight_scale, int32_t* ids, float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream) {
   if (rows <= 0) return 0;
   const size_t bytes = ((size_t)rows * (experts + 2 * groups) + (size_t)rows * top) * sizeof(float);
   if (rows > 16 || bytes > 48 * 1024) {
-    const int rc = bw_moe_route(logits, ld, rows, experts, top, groups, keep, ids, wts, stream);
+    const int rc = bw_moe_route(logits, ld, rows, experts, top, groups, keep, weight_scale, ids, wts, stream);
     return rc != 0 ? rc : bw_moe_plan(ids, rows * top, experts, sorted, place, tiles, meta, stream);
   }
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || groups < 1 || experts % groups || keep < 1 || keep > groups ||
       top > keep * (experts / groups))
     return -2;
   hipLaunchKernelGGL(moe_route_plan_kernel, dim3(1), dim3(1024), bytes, (hipStream_t)stream, logits, ld, rows, experts, top, groups, keep,
-                     ids, wts, 1024 / experts, bw_moe_tile_rows(rows * top), sorted, place, tiles, meta);
+                     weight_scale, ids, wts, 1024 / experts, bw_moe_tile_rows(rows * top), sorted, place, tiles, meta);
   return BW_LAUNCH_CHECK();
 }
 
 // ------------------------------------------------------------------------------ the experts' activation
 
 __device__ __forceinline__ float moe_act(float g, float u, float limit, float alpha) {
+  if (!(limit > 0.0f)) return (g * (1.0f / (1.0f + bw_expf(-alpha * g)))) * u;      // the plain gated form
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return (g * (1.0f / (1.0f + bw_expf(-alpha * g)))) * (u + 1.0f);

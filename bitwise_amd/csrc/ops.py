@@ -55,12 +55,12 @@ _SIGS = {
     "bw_gemm_qkv_rope_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_attention_f32_tiles": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p,
-                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p],
+                               c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_int, c_float, c_void_p],
     "bw_attention_f32": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p],
+                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_int, c_float, c_void_p],
     "bw_attention_bf16": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_longlong,
-                          c_void_p, c_int, c_void_p, c_void_p],
+                          c_void_p, c_int, c_void_p, c_int, c_float, c_void_p],
     "bw_attention_decode_scratch": [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "bw_attention_fold_group_tiles": [c_int],
     "bw_norm_gemm_supported": [c_int, c_int],
@@ -83,7 +83,12 @@ _SIGS = {
                              c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p],
     "bw_head_norm_gate": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_int, c_int, c_float, c_void_p],
-    "bw_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_glu": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p],
+    "bw_embed_sum": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                     c_float, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "bw_whole_norm_kv": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int,
+                         c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                         c_int, c_int, c_void_p],
     "bw_shared_key_attention_mfma": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
                                      c_void_p, c_longlong, c_void_p],
@@ -103,9 +108,10 @@ _SIGS = {
     "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
                     c_int, c_void_p],
     "bw_softcap": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
-    "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-    "bw_moe_route_plan": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_void_p],
+    "bw_scale_rows": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p],
+    "bw_moe_route_plan": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                          c_void_p, c_void_p],
     "bw_moe_max_tiles": [c_int, c_int],
     "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_moe_experts": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -180,6 +186,16 @@ def _need(t: torch.Tensor, dtype, what: str) -> None:
         raise ValueError(f"{what} must be contiguous")
 
 
+def _need_strided(t: torch.Tensor, dtype, what: str) -> None:
+    """As ``_need`` for a view whose rows lie a stride apart (the caller passes the stride on)."""
+    if not t.is_cuda:
+        raise ValueError(f"{what} must live on the GPU (there is no CPU path)")
+    if t.dtype != dtype:
+        raise ValueError(f"{what} must be {dtype}, got {t.dtype}")
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{what} must be a matrix whose rows are contiguous")
+
+
 def _is_bf16(t: torch.Tensor, what: str) -> int:
     if t.dtype == torch.bfloat16:
         return 1
@@ -251,6 +267,45 @@ def embed(tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, feedback
             raise ValueError("embed: feedback is shorter than the rows")
     _check(_fn("bw_embed")(tokens.data_ptr(), None if feedback is None else feedback.data_ptr(), table.data_ptr(),
                            _is_bf16(table, "table"), out.data_ptr(), rows, width, vocab, _stream()), "embed")
+
+
+def embed_sum(tokens: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, scale: float, out: torch.Tensor,
+              pair_table: Optional[torch.Tensor] = None, pair_hash: Tuple[int, int, int] = (0, 0, 0),
+              pos_table: Optional[torch.Tensor] = None, row_seq: Optional[torch.Tensor] = None,
+              seq_rows: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+              state: Optional[torch.Tensor] = None, feedback: Optional[torch.Tensor] = None) -> None:
+    """out[r] = table[token] * scale + pair_table[row] + pos_table[position], 32-bit, the two last tables optional.
+    ``pair_hash`` = (buckets, mul_prev, mul_cur): row = (token before * mul_prev + token * mul_cur) mod buckets, and row
+    ``buckets`` at a request's position 0.  The token before a request's first row of the step is ``state[slot]`` (int32, a
+    word a slot), which then takes the request's last token of the step.  Tokens as in ``embed``."""
+    _need(tokens, torch.int32, "tokens")
+    _need(positions, torch.int32, "positions")
+    _need(out, torch.float32, "out")
+    rows = tokens.numel()
+    vocab, width = table.shape
+    tables = [t for t in (table, pair_table, pos_table) if t is not None]
+    if any(not t.is_cuda or not t.is_contiguous() or t.dim() != 2 or t.shape[1] != width or t.dtype != table.dtype for t in tables):
+        raise ValueError("embed_sum: the tables must be contiguous GPU matrices of one dtype and one width")
+    if out.shape[0] < rows or out.shape[1] != width or positions.numel() < rows:
+        raise ValueError(f"embed_sum: out {tuple(out.shape)} or the positions do not fit {rows} rows of width {width}")
+    buckets, mul_prev, mul_cur = (int(v) for v in pair_hash)
+    if pair_table is not None:
+        for t, what in ((row_seq, "row_seq"), (seq_rows, "seq_rows"), (slots, "slots"), (state, "state")):
+            if t is None:
+                raise ValueError(f"embed_sum: a table of token pairs needs {what}")
+            _need(t, torch.int32, what)
+        if buckets < 1 or pair_table.shape[0] != buckets + 1 or row_seq.numel() < rows:
+            raise ValueError("embed_sum: the pair table has one row more than buckets")
+    if feedback is not None:
+        _need(feedback, torch.int32, "feedback")
+        if feedback.numel() < rows:
+            raise ValueError("embed_sum: feedback is shorter than the rows")
+    ptr = lambda t: 0 if t is None else t.data_ptr()
+    _check(_fn("bw_embed_sum")(tokens.data_ptr(), ptr(feedback), positions.data_ptr(), ptr(row_seq), ptr(seq_rows), ptr(slots),
+                               ptr(state), table.data_ptr(), ptr(pair_table), ptr(pos_table), _is_bf16(table, "table"),
+                               float(scale), buckets, mul_prev, mul_cur,
+                               0x7fffffff if pos_table is None else pos_table.shape[0], out.data_ptr(), rows, width, vocab,
+                               _stream()), "embed_sum")
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, rows: int, eps: float) -> None:
@@ -518,9 +573,11 @@ def _sink_ptr(sink: Optional[torch.Tensor], heads: int) -> int:
 def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
                   k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, rows: int, heads: int,
                   kv_heads: int, head_dim: int, page_size: int, window: int, scale: float,
-                  sink: Optional[torch.Tensor] = None) -> None:
+                  sink: Optional[torch.Tensor] = None, chunk: int = 0, softcap: float = 0.0) -> None:
     """q: [rows, stride] float32 with head h at columns h*head_dim.. (the stacked q|k|v rows
-    serve as they are); caches [pages, kv_heads, page_size, head_dim] float32."""
+    serve as they are); caches [pages, kv_heads, page_size, head_dim] float32.  ``chunk`` > 0: a query sees only the keys
+    of its own run of ``chunk`` positions counted from position 0 (instead of a window); ``softcap`` > 0: a score s
+    becomes softcap * tanh(s / softcap) before the softmax."""
     _need(q, torch.float32, "q")
     _need(out, torch.float32, "out")
     _need(k_cache, torch.float32, "k_cache")
@@ -537,13 +594,14 @@ def attention_f32(q: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tenso
     _check(_fn("bw_attention_f32")(q.data_ptr(), q.stride(0), positions.data_ptr(), row_seq.data_ptr(),
                                    block_table.data_ptr(), block_table.stride(0), k_cache.data_ptr(),
                                    v_cache.data_ptr(), out.data_ptr(), out.stride(0), rows, heads, kv_heads, head_dim,
-                                   page_size, int(window), float(scale), _sink_ptr(sink, heads), _stream()), "attention_f32")
+                                   page_size, int(window), float(scale), _sink_ptr(sink, heads), int(chunk), float(softcap),
+                                   _stream()), "attention_f32")
 
 
 def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
                         num_tiles: int, tiled, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                         heads: int, kv_heads: int, head_dim: int, page_size: int, window: int, scale: float,
-                        sink: Optional[torch.Tensor] = None) -> None:
+                        sink: Optional[torch.Tensor] = None, chunk: int = 0, softcap: float = 0.0) -> None:
     """``attention_f32`` over tiles ([tiles, 4] int32 = first row, rows, request, 0; a tile's rows are consecutive
     rows of one request).  ``tiled`` True (1): a workgroup per tile of up to 16 rows, keys and values shared
     through LDS; 2: a wave per tile of up to 32 rows, both products as chains of single-step matrix instructions
@@ -566,7 +624,7 @@ def attention_f32_tiles(q: torch.Tensor, positions: torch.Tensor, block_table: t
                                          block_table.stride(0), tiles.data_ptr(), int(num_tiles), int(tiled),
                                          k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), out.stride(0), heads,
                                          kv_heads, head_dim, page_size, int(window), float(scale), _sink_ptr(sink, heads),
-                                         _stream()),
+                                         int(chunk), float(softcap), _stream()),
            "attention_f32_tiles")
 
 
@@ -574,7 +632,8 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
                    tiles: Optional[torch.Tensor], num_tiles: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    out: torch.Tensor, heads: int, kv_heads: int, head_dim: int, page_size: int, window: int,
                    scale: float, decode: bool = False,
-                   scratch: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, sink: Optional[torch.Tensor] = None) -> None:
+                   scratch: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, sink: Optional[torch.Tensor] = None,
+                   chunk: int = 0, softcap: float = 0.0) -> None:
     """q, out: [rows, heads*head_dim] bfloat16; k pages [kv_heads, page, hd], v pages
     [kv_heads, hd, page]; tiles int32 [n, 4] = (first row, tokens, sequence, 0).
 
@@ -623,7 +682,7 @@ def attention_bf16(q: torch.Tensor, positions: torch.Tensor, block_table: torch.
                                     out.stride(0), heads, kv_heads, head_dim, page_size, int(window), float(scale), int(decode),
                                     sc_f.data_ptr() if sc_f is not None else 0, sc_f.numel() if sc_f is not None else 0,
                                     sc_c.data_ptr() if sc_c is not None else 0, sc_c.numel() if sc_c is not None else 0,
-                                    _sink_ptr(sink, heads), _stream()),
+                                    _sink_ptr(sink, heads), int(chunk), float(softcap), _stream()),
            "attention_bf16")
 
 
@@ -687,7 +746,7 @@ def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor
 RECUR_DECAY_PER_CHANNEL, RECUR_SCALAR_GATES = 0, 1
 RECUR_MAX_DIM = 256          # key channels of a head that the recurrence keeps in a lane's registers
 GATE_SIGMOID, GATE_SILU = 0, 1
-ACT_SILU, ACT_GELU_TANH = 0, 1
+ACT_SILU, ACT_GELU_TANH, ACT_CLAMPED_SWISH = 0, 1, 2
 
 
 def _act_out(t: torch.Tensor, what: str) -> int:
@@ -797,13 +856,24 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, per_head_weight: bool,
                                     heads, vdim, float(eps), _stream()), "head_norm_gate")
 
 
-def glu(gate_up: torch.Tensor, out: torch.Tensor, rows: int, act: int) -> None:
-    """out = act(gate) * up of the stacked 32-bit product [rows, 2*inter]; out float32 or bfloat16 (one rounding)."""
+def glu(gate_up: torch.Tensor, out: torch.Tensor, rows: int, act: int, limit: float = 0.0, alpha: float = 1.0,
+        row_gate: Optional[torch.Tensor] = None) -> None:
+    """out = act(gate) * up of the stacked 32-bit product [rows, >= 2*inter] (gate at column 0, up at column inter); out
+    float32 or bfloat16 (one rounding).  ACT_CLAMPED_SWISH: g = min(gate, limit), u = clamp(up, -limit, limit),
+    out = g sigmoid(alpha g) (u + 1).  ``row_gate`` (a 32-bit column, one number a row): out's row r is multiplied by
+    sigmoid(row_gate[r])."""
     _need(gate_up, torch.float32, "gate_up")
     inter = out.shape[1]
-    if gate_up.shape[1] != 2 * inter or gate_up.shape[0] < rows or out.shape[0] < rows:
+    if gate_up.shape[1] < 2 * inter or gate_up.shape[0] < rows or out.shape[0] < rows:
         raise ValueError("glu: gate_up must be [rows, 2*inter] for out [rows, inter]")
-    _check(_fn("bw_glu")(gate_up.data_ptr(), out.data_ptr(), _act_out(out, "out"), rows, inter, int(act), _stream()), "glu")
+    rg, ldrg = 0, 0
+    if row_gate is not None:
+        _need_strided(row_gate, torch.float32, "row_gate")
+        if row_gate.dim() != 2 or row_gate.shape[1] != 1 or row_gate.shape[0] < rows:
+            raise ValueError("glu: row_gate must be a column [rows, 1]")
+        rg, ldrg = row_gate.data_ptr(), row_gate.stride(0)
+    _check(_fn("bw_glu")(gate_up.data_ptr(), gate_up.stride(0), out.data_ptr(), _act_out(out, "out"), rows, inter, int(act),
+                         float(limit), float(alpha), rg, ldrg, _stream()), "glu")
 
 
 # ------------------------------------------------------------------------------ attention over a compressed cache
@@ -1025,6 +1095,51 @@ def pair_rope_unit(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Te
                                     int(has_kv), int(write_cache and has_kv), _stream()), "pair_rope_unit")
 
 
+def whole_norm_kv(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
+                  q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float, q_out: torch.Tensor, k_cache: torch.Tensor,
+                  v_cache: torch.Tensor, rows: int, heads: int, kv_heads: int, dim: int, vdim: int, head_size: int,
+                  page_size: int, write_cache: bool, v_first: Optional[torch.Tensor] = None,
+                  mix: Optional[torch.Tensor] = None, v_keep: Optional[torch.Tensor] = None) -> None:
+    """Queries and keys of ``src`` [rows, q | k | v] (32-bit) normed over their whole projection, all heads at once,
+    x / sqrt(mean(x^2) + eps) * weight; the queries go to ``q_out`` [rows, heads * head_size] and keys and values into
+    the row's place in the paged cache, heads padded with zeros to ``head_size``.  ``v_first`` [rows, kv_heads * vdim]
+    (32-bit) with ``mix`` (one 32-bit number on the device): the values are stored as (1 - mix) v + mix v_first.
+    ``v_keep``: receives the values as projected."""
+    _need(src, torch.float32, "src")
+    _need(q_weight, torch.float32, "q_weight")
+    _need(k_weight, torch.float32, "k_weight")
+    for t, what in ((positions, "positions"), (row_seq, "row_seq"), (block_table, "block_table")):
+        _need(t, torch.int32, what)
+    is_bf16 = _act_out(q_out, "q_out")
+    if k_cache.dtype != q_out.dtype or v_cache.dtype != q_out.dtype:
+        raise ValueError("whole_norm_kv: the queries and the cache have one dtype")
+    if src.shape[0] < rows or q_out.shape[0] < rows or q_out.shape[1] != heads * head_size:
+        raise ValueError("whole_norm_kv: src or q_out do not fit")
+    if q_weight.numel() != heads * dim or k_weight.numel() != kv_heads * dim:
+        raise ValueError("whole_norm_kv: the norms' weights cover the whole projections")
+    if src.shape[1] < heads * dim + (kv_heads * (dim + vdim) if write_cache else 0):
+        raise ValueError("whole_norm_kv: src is narrower than the projections")
+    page_elems = kv_heads * page_size * head_size
+    if k_cache.shape[-1] != page_elems or v_cache.shape[-1] != page_elems:
+        raise ValueError("whole_norm_kv: the cache's pages do not fit")
+    for t, what in ((v_first, "v_first"), (v_keep, "v_keep")):
+        if t is not None:
+            _need(t, torch.float32, what)
+            if t.shape[0] < rows or t.shape[1] < kv_heads * vdim:
+                raise ValueError(f"whole_norm_kv: {what} does not fit")
+    if v_first is not None:
+        if mix is None:
+            raise ValueError("whole_norm_kv: mixing needs its weight")
+        _need(mix, torch.float32, "mix")
+    ptr = lambda t: 0 if t is None else t.data_ptr()
+    ld = lambda t: 0 if t is None else t.stride(0)
+    _check(_fn("bw_whole_norm_kv")(src.data_ptr(), src.stride(0), positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
+                                   block_table.stride(0), q_weight.data_ptr(), k_weight.data_ptr(), float(eps), ptr(v_first),
+                                   ld(v_first), ptr(mix) if v_first is not None else 0, ptr(v_keep), ld(v_keep), q_out.data_ptr(),
+                                   k_cache.data_ptr(), v_cache.data_ptr(), is_bf16, rows, heads, kv_heads, dim, vdim, head_size,
+                                   page_size, int(bool(write_cache)), _stream()), "whole_norm_kv")
+
+
 def gate_mul(av: torch.Tensor, head_size: int, g: torch.Tensor, out: torch.Tensor, rows: int, heads: int, vdim: int) -> None:
     """out[r, h*vdim + d] = av[r, h*head_size + d] * sigmoid(g[r, h*vdim + d]); ``g`` float32 (a column slice will do)."""
     if g.dtype != torch.float32 or g.stride(1) != 1 or g.shape[1] < heads * vdim:
@@ -1106,6 +1221,14 @@ def softcap(x: torch.Tensor, rows: int, cap: float) -> None:
     _check(_fn("bw_softcap")(x.data_ptr(), x.stride(0), rows, x.shape[1], float(cap), _stream()), "softcap")
 
 
+def scale_rows(x: torch.Tensor, rows: int, factor: float) -> None:
+    """x[:rows] *= factor in place (32-bit)."""
+    _need(x, torch.float32, "x")
+    if x.shape[0] < rows:
+        raise ValueError("scale_rows: fewer rows than said")
+    _check(_fn("bw_scale_rows")(x.data_ptr(), x.stride(0), rows, x.shape[1], float(factor), _stream()), "scale_rows")
+
+
 # ------------------------------------------------------------------------------ routed experts
 
 def moe_max_tiles(slots: int, experts: int) -> int:
@@ -1113,20 +1236,21 @@ def moe_max_tiles(slots: int, experts: int) -> int:
     return int(_fn("bw_moe_max_tiles")(int(slots), int(experts)))
 
 
-def moe_route(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor) -> None:
+def moe_route(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor,
+              weight_scale: float = 1.0, experts: Optional[int] = None) -> None:
     """Per row: softmax over the experts' logits; the ``top`` best experts among those of the ``keep`` best of ``groups``
     equal groups of neighbours (a group's score: its best expert's); ``ids`` [rows, top] int32 in the order chosen,
     ``wts`` [rows, top] their scores."""
     _need(logits, torch.float32, "logits")
     _need(ids, torch.int32, "ids")
     _need(wts, torch.float32, "wts")
-    experts = logits.shape[1]
-    if logits.shape[0] < rows or ids.numel() < rows * top or wts.numel() < rows * top:
+    experts = logits.shape[1] if experts is None else int(experts)      # (the rows may hold more columns behind the experts')
+    if logits.shape[0] < rows or logits.shape[1] < experts or ids.numel() < rows * top or wts.numel() < rows * top:
         raise ValueError("moe_route: buffers shorter than the rows")
     if experts % groups or not 1 <= keep <= groups or not 1 <= top <= keep * (experts // groups):
         raise ValueError("moe_route: groups, keep and top do not fit the experts")
-    _check(_fn("bw_moe_route")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, ids.data_ptr(),
-                               wts.data_ptr(), _stream()), "moe_route")
+    _check(_fn("bw_moe_route")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, float(weight_scale),
+                               ids.data_ptr(), wts.data_ptr(), _stream()), "moe_route")
 
 
 def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor,
@@ -1141,20 +1265,24 @@ def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Te
 
 
 def moe_route_plan(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor,
-                   sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor, meta: torch.Tensor) -> None:
-    """``moe_route`` followed by ``moe_plan`` over the rows' choices; steps of up to 16 rows do both in one launch."""
+                   sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor, meta: torch.Tensor,
+                   weight_scale: float = 1.0, experts: Optional[int] = None) -> None:
+    """``moe_route`` followed by ``moe_plan`` over the rows' choices; steps of up to 16 rows do both in one launch.
+    ``weight_scale``: the chosen scores are multiplied by it; ``experts``: the leading columns of ``logits`` that are the
+    experts' (all of them by default)."""
     _need(logits, torch.float32, "logits")
     _need(wts, torch.float32, "wts")
     for t, what in ((ids, "ids"), (sorted_slots, "sorted"), (place, "place"), (tiles, "tiles"), (meta, "meta")):
         _need(t, torch.int32, what)
-    experts, slots = logits.shape[1], rows * top
-    if logits.shape[0] < rows or min(ids.numel(), wts.numel(), sorted_slots.numel(), place.numel()) < slots:
+    experts, slots = (logits.shape[1] if experts is None else int(experts)), rows * top
+    if logits.shape[0] < rows or logits.shape[1] < experts or min(ids.numel(), wts.numel(), sorted_slots.numel(), place.numel()) < slots:
         raise ValueError("moe_route_plan: buffers shorter than the rows")
     if experts % groups or not 1 <= keep <= groups or not 1 <= top <= keep * (experts // groups):
         raise ValueError("moe_route_plan: groups, keep and top do not fit the experts")
     if tiles.numel() < 4 * moe_max_tiles(slots, experts) or meta.numel() < 1:
         raise ValueError("moe_route_plan: the plan's tables are too small")
-    _check(_fn("bw_moe_route_plan")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, ids.data_ptr(), wts.data_ptr(),
+    _check(_fn("bw_moe_route_plan")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, float(weight_scale),
+                                    ids.data_ptr(), wts.data_ptr(),
                                     sorted_slots.data_ptr(), place.data_ptr(), tiles.data_ptr(), meta.data_ptr(), _stream()),
            "moe_route_plan")
 

@@ -472,23 +472,30 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 
 // ------------------------------------------------------------------------- gated unit
 
-enum { ACT_SILU = 0, ACT_GELU_TANH = 1 };
+enum { ACT_SILU = 0, ACT_GELU_TANH = 1, ACT_CLAMPED_SWISH = 2 };
 
 template <typename OT>
-__global__ void glu_kernel(const float* __restrict__ gu, OT* __restrict__ hout, long long n, int inter, int act) {
+__global__ void glu_kernel(const float* __restrict__ gu, int ldg, OT* __restrict__ hout, long long n, int inter, int act, float limit,
+                           float alpha, const float* __restrict__ row_gate, int ld_row_gate) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const long long row = idx / inter;
   const int c = (int)(idx % inter);
-  const float g = gu[row * 2 * inter + c], u = gu[row * 2 * inter + inter + c];
+  float g = gu[row * ldg + c], u = gu[row * ldg + inter + c];
   float ag;
   if (act == ACT_GELU_TANH) {
     const float inner = 0.7978845608028654f * (g + 0.044715f * ((g * g) * g));
     ag = (0.5f * g) * (1.0f + tanhf(inner));
+  } else if (act == ACT_CLAMPED_SWISH) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit) + 1.0f;
+    ag = g * (1.0f / (1.0f + bw_expf(-alpha * g)));
   } else {
     ag = g * (1.0f / (1.0f + bw_expf(-g)));
   }
-  store_act(hout + idx, ag * u);
+  float h = ag * u;
+  if (row_gate != nullptr) h *= 1.0f / (1.0f + bw_expf(-row_gate[row * ld_row_gate]));
+  store_act(hout + idx, h);
 }
 
 }  // namespace
@@ -548,13 +555,15 @@ extern "C" int bw_head_norm_gate(const float* o, int ldi, const float* weight, i
   return BW_LAUNCH_CHECK();
 }
 
-extern "C" int bw_glu(const float* gate_up, void* h, int out_is_bf16, int rows, int inter, int act, void* stream) {
+extern "C" int bw_glu(const float* gate_up, int ldg, void* h, int out_is_bf16, int rows, int inter, int act, float limit, float alpha,
+                      const float* row_gate, int ld_row_gate, void* stream) {
   if (rows <= 0 || inter <= 0) return 0;
-  if (act != ACT_SILU && act != ACT_GELU_TANH) return -2;
+  if (act != ACT_SILU && act != ACT_GELU_TANH && act != ACT_CLAMPED_SWISH) return -2;
+  if (ldg < 2 * inter || (act == ACT_CLAMPED_SWISH && !(limit > 0.0f))) return -2;
   const long long n = (long long)rows * inter;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-  if (out_is_bf16) hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, block, 0, s, gate_up, (bf16_t*)h, n, inter, act);
-  else hipLaunchKernelGGL(glu_kernel<float>, grid, block, 0, s, gate_up, (float*)h, n, inter, act);
+  if (out_is_bf16) hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, block, 0, s, gate_up, ldg, (bf16_t*)h, n, inter, act, limit, alpha, row_gate, ld_row_gate);
+  else hipLaunchKernelGGL(glu_kernel<float>, grid, block, 0, s, gate_up, ldg, (float*)h, n, inter, act, limit, alpha, row_gate, ld_row_gate);
   return BW_LAUNCH_CHECK();
 }

@@ -39,8 +39,9 @@ class StepContext:
     """
 
     def __init__(self, segments: Sequence[Segment], num_groups: int, ws, calls: Sequence[Any] = (),
-                 num_pages: Optional[int] = None):
+                 num_pages: Optional[int] = None, embedding_state: Optional[torch.Tensor] = None):
         given = list(segments)
+        self.embedding_state = embedding_state       # the engine's per-slot state of the model's embedding, if it keeps one
 
         def rank(i: int):
             n = len(given[i].tokens)

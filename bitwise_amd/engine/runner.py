@@ -36,8 +36,9 @@ class _StaticDecodeContext:
     one_row_per_request = True                           # row t is the one token of request t
     wants_every_row = True                               # row i is wanted place i: the model need not gather
 
-    def __init__(self, size: int, num_groups: int, max_pages: int, ws: Workspace, calls, num_pages: int):
+    def __init__(self, size: int, num_groups: int, max_pages: int, ws: Workspace, calls, num_pages: int, embedding_state=None):
         self.rows = self.nseq = self.num_wanted = size
+        self.embedding_state = embedding_state
         self.ws, self.calls = ws, list(calls)
         self.device = device = ws.device
         self.page_size = ws.page_size
@@ -187,7 +188,8 @@ class ModelRunner:
         return self.model.forward(self._context(segments))
 
     def _context(self, segments: Sequence[Segment]) -> StepContext:
-        return StepContext(segments, len(self.model.group_specs), self.ws, self.storage.bindings, self.storage.num_pages)
+        return StepContext(segments, len(self.model.group_specs), self.ws, self.storage.bindings, self.storage.num_pages,
+                           embedding_state=self.storage.embedding_state)
 
     def check_phases(self, bits: Optional[int] = None) -> None:
         """Raise if a wait inside one of the launches of several phases gave up since the last check.  ``bits``: the
@@ -224,7 +226,7 @@ class ModelRunner:
         ws = self.ws
         max_pages = (self.max_model_len + ws.page_size - 1) // ws.page_size
         ctx = _StaticDecodeContext(bucket, len(self.model.group_specs), max_pages, ws, self.storage.bindings,
-                                   self.storage.num_pages)
+                                   self.storage.num_pages, embedding_state=self.storage.embedding_state)
         # One eager run first, on rows that are all padding: it creates every scratch buffer the capture
         # will use and touches neither cache nor state (a real step run here and then replayed from the
         # fresh graph would advance a stateful mixer twice).

@@ -36,6 +36,10 @@ class CacheStorage:
         self.block_states: Dict[int, torch.Tensor] = {}
         for idx, ss in model.block_state_specs.items():
             self.block_states[idx] = torch.zeros((self.num_slots, *ss.shape), dtype=_TORCH_DTYPE[ss.dtype], device=rt.device)
+        # the embedding's own per-request state (the token before), a row per slot
+        es = model.embedding_state_spec
+        self.embedding_state = None if es is None else torch.zeros((self.num_slots, *es.shape), dtype=_TORCH_DTYPE[es.dtype],
+                                                                     device=rt.device)
         self.bindings: List[CallBinding] = []
         for plan in model.calls:
             call = dataclasses.replace(plan, state=self.states.get(plan.index), block_state=self.block_states.get(plan.index))
@@ -46,6 +50,8 @@ class CacheStorage:
 
     def nbytes(self) -> int:
         tensors = self.keys + self.values + list(self.states.values()) + list(self.block_states.values())
+        if self.embedding_state is not None:
+            tensors.append(self.embedding_state)
         return sum(t.numel() * t.element_size() for t in tensors)
 
     def bytes_per_token(self) -> int:
@@ -59,6 +65,8 @@ class CacheStorage:
         """Fixed-size state starts from zero when a request takes the slot."""
         for t in list(self.states.values()) + list(self.block_states.values()):
             t[slot].zero_()
+        if self.embedding_state is not None:
+            self.embedding_state[slot].zero_()
 
     def poison_pages(self, group: int, pages) -> None:
         """Fill the given pages of a group, in all its caches, with NaN (tests: a page that is

@@ -51,6 +51,7 @@ class AssembledModel:
         self.final_norm = lookup(base.NORMS, "norm", spec.final_norm.kind)(spec.final_norm.params, runtime)
         self.lm_head = lookup(base.HEADS, "head", spec.lm_head.kind)(spec.lm_head.params, runtime)
         self._plan_caches(spec.schedule)
+        self.embedding_state_spec: Optional[StateSpec] = self.embedding.state_spec()
         every = [self.embedding, self.final_norm, self.lm_head] + [p for b in self.layers for p in (b, *b.parts.values())]
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in every)
         # (a captured decode step may hold its launches back to join them only if none of them goes round ops)
@@ -58,13 +59,14 @@ class AssembledModel:
         # each mixer's own word on what the engine may do around it (parts.base.Mixer)
         mixers = [self.layers[c.layer].mixer for c in spec.schedule]
         stateless_blocks = not self.block_state_specs
-        self.prefix_reusable = stateless_blocks and all(m.prefix_reusable for m in mixers)
+        # (an embedding's state is the token before: a request that starts behind another's pages would not have it)
+        self.prefix_reusable = stateless_blocks and self.embedding_state_spec is None and all(m.prefix_reusable for m in mixers)
         self.run_ahead_safe = stateless_blocks and all(m.run_ahead_safe for m in mixers)
 
     @property
     def has_state(self) -> bool:
         """Whether a request holds anything outside its pages (a slot of some mixer's or arrangement's state)."""
-        return bool(self.state_specs or self.block_state_specs)
+        return bool(self.state_specs or self.block_state_specs or self.embedding_state_spec is not None)
 
     def check_page_size(self, page_size: int) -> None:
         """Refuse a page size that one of the mixers' kernels does not take."""

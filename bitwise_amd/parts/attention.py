@@ -79,13 +79,24 @@ def _split_scratch(ws, tiles: int, table_width: int, heads: int, kv_heads: int, 
     return sizes
 
 
-def attend_bf16(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None) -> None:
+def _mask_and_cap(sink, chunk: int, softcap: float) -> dict:
+    extra = {} if sink is None else {"sink": sink}
+    if chunk:
+        extra["chunk"] = int(chunk)
+    if softcap:
+        extra["softcap"] = float(softcap)
+    return extra
+
+
+def attend_bf16(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None,
+                chunk: int = 0, softcap: float = 0.0) -> None:
     """bfloat16 attention over the call's cache for the step's queries ``q`` [rows, heads*head_dim] into ``out`` (the same
     shape): prompt portions through the fold kernel, decoded tokens with long contexts through the decode kernel.
-    ``sink`` [heads]: a score per head that joins the denominator and has no value."""
+    ``sink`` [heads]: a score per head that joins the denominator and has no value.  ``chunk``: a query sees the keys of
+    its own run of that many positions only; ``softcap``: scores are squashed to cap * tanh(s / cap)."""
     ws = ctx.ws
     table = ctx.block_tables[call.group]
-    extra = {} if sink is None else {"sink": sink}
+    extra = _mask_and_cap(sink, chunk, softcap)
     tokens_per_tile = 16 // min(heads // kv_heads, 16)
     plan = plan_tiles(ctx, tokens_per_tile, ops.fold_group_tiles(head_dim))
     common = (call.k_cache, call.v_cache, out, heads, kv_heads, head_dim, ws.page_size, window, scale)
@@ -104,12 +115,13 @@ def attend_bf16(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, win
                            scratch=scratch, **extra)
 
 
-def attend_f32(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None) -> None:
+def attend_f32(ctx, call, q, out, heads: int, kv_heads: int, head_dim: int, window: int, scale: float, sink=None,
+               chunk: int = 0, softcap: float = 0.0) -> None:
     """32-bit attention over the call's cache: ``q`` [rows, >= heads*head_dim] with head h at h*head_dim, ``out``
-    [rows, heads*head_dim]."""
+    [rows, heads*head_dim].  ``chunk``, ``softcap``: as ``attend_bf16``."""
     ws, rows = ctx.ws, ctx.rows
     table = ctx.block_tables[call.group]
-    extra = {} if sink is None else {"sink": sink}
+    extra = _mask_and_cap(sink, chunk, softcap)
     # prompt portions: tiles of 32 rows, a wave a tile, both products on the matrix cores; for head sizes
     # that fill the second product's blocks badly (80 to 112) tiles of 16 rows on the vector units
     on_matrix_cores = head_dim <= 64 or head_dim == 128

@@ -147,6 +147,11 @@ class Part:
 
 
 class Embedding(Part):
+    def state_spec(self) -> Optional["StateSpec"]:
+        """Per-request state of an embedding that looks at the token before (None: it has none).  The bound tensor, a row
+        per slot, arrives as ``ctx.embedding_state``."""
+        return None
+
     def forward(self, ctx):
         """Token ids ``ctx.tokens`` -> the 32-bit residual stream [max_rows, width] (a buffer of
         the context's workspace; rows of negative tokens are zero)."""

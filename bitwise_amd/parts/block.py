@@ -10,16 +10,25 @@ from .base import Block, register_block
 
 @register_block("prenorm")
 class PreNormBlock(Block):
-    """x += mixer(norm1(x)); x += feed_forward(norm2(x)) (src/model.cpp:281-305)."""
+    """x += mixer(norm1(x)); x += feed_forward(norm2(x)) (src/model.cpp:281-305).  A layer may leave the feed-forward
+    (and its norm) out."""
 
     roles = {"mixer_norm": "norm", "ffn_norm": "norm", "mixer": "mixer", "feed_forward": "feed_forward"}
+    optional_roles = ("ffn_norm", "feed_forward")
     graph_safe = True
     launches_through_ops = True
+
+    def __init__(self, parts, runtime):
+        super().__init__(parts, runtime)
+        if (self.feed_forward is None) != (self.ffn_norm is None):
+            raise ValueError("prenorm block: a feed-forward and its norm come together or not at all")
 
     def forward(self, ctx, call, x) -> None:
         if not self.mixer.forward_with_norm(ctx, call, x, self.mixer_norm, x):
             h = self.mixer_norm.forward(ctx, x)
             self.mixer.forward(ctx, call, h, x)
+        if self.feed_forward is None:
+            return
         if not self.feed_forward.forward_with_norm(ctx, x, self.ffn_norm, x):
             h = self.ffn_norm.forward(ctx, x)
             self.feed_forward.forward(ctx, h, x)

@@ -7,7 +7,7 @@ from typing import Dict, Optional
 import torch
 
 from ..csrc import ops
-from .base import Embedding, Head, TensorSpec, register_embedding, register_head
+from .base import Embedding, Head, StateSpec, TensorSpec, register_embedding, register_head
 from .linear import Linear
 
 
@@ -40,10 +40,68 @@ class TokenEmbedding(Embedding):
         return x
 
 
+@register_embedding("embedding_sum")
+class SummedEmbedding(TokenEmbedding):
+    """The token's row times a scale, plus (each optional) a row of a table of token pairs and a learned row per position:
+
+        x = table[token] * scale + pairs[(token before * mul_prev + token * mul_cur) mod buckets] + positions[p]
+
+    A request's first token takes the pair table's last row (number ``buckets``).  The token before a step's first token
+    of a request is per-request state (one word), so that a prompt may be cut anywhere.  All 32-bit.
+    params: vocab, width, tensor, scale (1); ``pairs``: None or {tensor, buckets, mul_prev, mul_cur}; ``positions``: None or
+    {tensor, count}."""
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.scale = float(params.get("scale", 1.0))
+        self.pairs = dict(params["pairs"]) if params.get("pairs") else None
+        self.positions = dict(params["positions"]) if params.get("positions") else None
+        if self.pairs is not None:
+            b, mp, mc = int(self.pairs["buckets"]), int(self.pairs["mul_prev"]), int(self.pairs["mul_cur"])
+            if b < 1 or mp < 0 or mc < 0:
+                raise ValueError("embedding_sum: the pair table needs at least one bucket and multipliers that are not negative")
+            self.pair_hash = (b, mp, mc)
+        self.pair_table = self.pos_table = None
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = super().tensors()
+        if self.pairs is not None:
+            out[str(self.pairs["tensor"])] = TensorSpec((self.pair_hash[0] + 1, self.width), "embedding")
+        if self.positions is not None:
+            out[str(self.positions["tensor"])] = TensorSpec((int(self.positions["count"]), self.width), "embedding")
+        return out
+
+    def bind(self, tensors) -> None:
+        super().bind(tensors)
+        put = lambda t: t.to(self.rt.device).to(self.weight.dtype).contiguous()     # (one dtype for the kernel; the same values)
+        if self.pairs is not None:
+            self.pair_table = put(tensors[str(self.pairs["tensor"])])
+        if self.positions is not None:
+            self.pos_table = put(tensors[str(self.positions["tensor"])])
+        stored = {t.dtype for t in tensors.values()}
+        if len(stored) != 1:
+            raise ValueError("embedding_sum: the tables must be stored in one dtype")
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return StateSpec((1,), "int32") if self.pairs is not None else None
+
+    def forward(self, ctx) -> torch.Tensor:
+        x = ctx.ws.buffer("residual", self.width, torch.float32)
+        state = getattr(ctx, "embedding_state", None)
+        if self.pairs is not None and state is None:
+            raise ValueError("embedding_sum: the step's context carries no state for the embedding (the token before)")
+        ops.embed_sum(ctx.tokens[:ctx.rows], ctx.positions, self.weight, self.scale, x,
+                      pair_table=self.pair_table, pair_hash=self.pair_hash if self.pairs is not None else (0, 0, 0),
+                      pos_table=self.pos_table, row_seq=ctx.row_seq, seq_rows=ctx.seq_rows, slots=ctx.slots, state=state,
+                      feedback=getattr(ctx, "token_feedback", None))
+        return x
+
+
 @register_head("lm_head")
 class LMHead(Head):
-    """params: vocab, width, tied.  tensor: weight [vocab, width] unless tied to the embedding
-    (src/model.cpp:170-171).  Only the wanted rows are normed and projected."""
+    """params: vocab, width, tied; optional ``scale``: the logits are multiplied by it (one 32-bit product each).
+    tensor: weight [vocab, width] unless tied to the embedding (src/model.cpp:170-171).  Only the wanted rows are normed
+    and projected."""
 
     graph_safe = True
     launches_through_ops = True
@@ -52,6 +110,7 @@ class LMHead(Head):
         super().__init__(params, runtime)
         self.vocab, self.width, self.tied = int(params["vocab"]), int(params["width"]), bool(params["tied"])
         self.tensor = str(params.get("tensor", "weight"))
+        self.scale = float(params.get("scale", 1.0))
         self.linear: Optional[Linear] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
@@ -77,9 +136,11 @@ class LMHead(Head):
         if (self.rt.bf16 and isinstance(norm, RMSNorm) and self.linear.mfma
                 and ops.can_fuse_norm(count, self.linear.weight, x)):
             ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.linear.weight, logits, count, ops.EPI_F32)
-            return logits
-        normed = norm.forward(ctx, x, out_name="final_normed", rows=count)
-        self.linear.store(ws, normed, logits, count)
+        else:
+            normed = norm.forward(ctx, x, out_name="final_normed", rows=count)
+            self.linear.store(ws, normed, logits, count)
+        if self.scale != 1.0:
+            ops.scale_rows(logits, count, self.scale)
         return logits
 
 

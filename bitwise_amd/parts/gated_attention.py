@@ -11,7 +11,17 @@ Every step is switched by a parameter, so that another design can take what it n
 convolution tensor: none), ``qk_norm``, ``sink`` (None, or a number that every head uses), ``gate``, ``shared_kv``
 (no key and value tensors: the call reads the cache of the layer the schedule names), query/key size ``dim`` and value
 size ``vdim`` (the cache's head size is the larger of the two, rounded up to what the attention kernels take; the
-padding is zeros).  The last taps - 1 projected rows of a request are its state.  Convolution, rotation, norms, scores
+padding is zeros).  Further switches:
+
+    position None          no rotation: positions do not enter the scores
+    qk_norm "whole"        q and k are normed over their whole projection, all heads at once, with learned weights
+                           (tensors q.norm, k.norm): x / sqrt(mean(x^2) + eps) * w
+    softcap c              s_j <- c tanh(s_j / c) before the softmax
+    chunk C                the query at position i sees key j <= i only if floor(i / C) = floor(j / C), positions counted
+                           from the request's first token (not together with a window)
+    v_mix "source"/"mix"   the first such layer of a model keeps its values of the step's rows ("source"); a later one
+                           ("mix") caches v <- (1 - lambda) v + lambda v_source, lambda the tensor ``vmix`` (one number)
+  The last taps - 1 projected rows of a request are its state.  Convolution, rotation, norms, scores
 and softmax are 32-bit in both modes; the cache, the queries and the gated output have the mode's activation dtype.
 """
 
@@ -51,7 +61,17 @@ class GatedAttention(Mixer):
         self.dim, self.vdim = int(p["dim"]), int(p["vdim"])
         self.scale, self.eps = float(p["scale"]), float(p.get("eps", 0.0))
         self.taps = int(p.get("conv") or 0)
+        self.whole_norm = p.get("qk_norm") == "whole"
         self.qk_norm, self.gate, self.shared_kv = bool(p.get("qk_norm", False)), bool(p.get("gate", False)), bool(p.get("shared_kv", False))
+        self.softcap = float(p.get("softcap") or 0.0)
+        self.chunk = int(p.get("chunk") or 0)
+        self.v_mix = p.get("v_mix") or None
+        if self.v_mix not in (None, "source", "mix"):
+            raise ValueError(f"gated_attention: v_mix is 'source' or 'mix', not {self.v_mix!r}")
+        if self.v_mix is not None and (self.shared_kv or not self.whole_norm):
+            raise ValueError("gated_attention: values are mixed by the kernel that norms whole projections, in layers with values of their own")
+        if self.softcap < 0 or self.chunk < 0 or (self.chunk and p.get("window")):
+            raise ValueError("gated_attention: a soft cap and a chunk are positive; a chunk does not go with a window")
         self.sink_value: Optional[float] = None if p.get("sink") is None else float(p["sink"])
         self.window: Optional[int] = p.get("window")
         if self.heads % self.kv_heads:
@@ -65,11 +85,16 @@ class GatedAttention(Mixer):
         if not fits:
             raise ValueError(f"gated_attention: heads of {need} elements; the attention kernels take up to {ops.HEAD_DIMS[-1]}")
         self.head_size = fits[0]                       # the cache's head size
-        pos = p["position"]
-        self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
-        if getattr(self.position, "layout", None) != "pairs":
-            raise ValueError(f"gated_attention rotates neighbouring pairs; position encoding '{pos.kind}' is laid out otherwise")
-        self.rot = int(self.position.rotary_dim)
+        pos = p.get("position")
+        self.position = None
+        self.rot = 0
+        if pos is not None:
+            self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
+            if getattr(self.position, "layout", None) != "pairs":
+                raise ValueError(f"gated_attention rotates neighbouring pairs; position encoding '{pos.kind}' is laid out otherwise")
+            self.rot = int(self.position.rotary_dim)
+        if self.whole_norm and self.rot:
+            raise ValueError("gated_attention: the norm over whole projections comes without rotation")
         if self.rot > self.dim:
             raise ValueError(f"gated_attention: {self.rot} rotated elements in heads of {self.dim}")
         self.q_ch = self.heads * self.dim
@@ -79,6 +104,7 @@ class GatedAttention(Mixer):
         self.proj: Optional[Linear] = None
         self.o: Optional[Linear] = None
         self.conv_w = self.sink = self.cos = self.sin = None
+        self.q_norm_w = self.k_norm_w = self.mix_w = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
         out = {"q": TensorSpec((self.q_ch, self.width))}
@@ -90,20 +116,34 @@ class GatedAttention(Mixer):
             if not self.shared_kv:
                 out["k.conv"] = TensorSpec((self.kv_heads * self.dim, self.taps), "conv")
                 out["v.conv"] = TensorSpec((self.kv_heads * self.vdim, self.taps), "conv")
+        if self.whole_norm:
+            out["q.norm"] = TensorSpec((self.q_ch,), "norm")
+            if not self.shared_kv:
+                out["k.norm"] = TensorSpec((self.kv_heads * self.dim,), "norm")
+        if self.v_mix is not None:
+            out["vmix"] = TensorSpec((), "unit_interval")      # (read by "mix" layers; a "source" layer's is stored and unused)
         if self.gate:
             out["g"] = TensorSpec((self.g_ch, self.width))
         out["o"] = TensorSpec((self.width, self.heads * self.vdim))
         return out
 
     def bind(self, tensors) -> None:
-        self.cos, self.sin = self.position.tables()
+        dev = self.rt.device
+        if self.position is not None:
+            self.cos, self.sin = self.position.tables()
+        else:
+            self.cos = self.sin = torch.zeros(1, dtype=torch.float32, device=dev)      # (never read: nothing is rotated)
+        if self.whole_norm:
+            self.q_norm_w = tensors["q.norm"].to(dev).float().contiguous()            # (widening is exact)
+            self.k_norm_w = self.q_norm_w if self.shared_kv else tensors["k.norm"].to(dev).float().contiguous()
+        if self.v_mix == "mix":
+            self.mix_w = tensors["vmix"].to(dev).float().reshape(1).contiguous()
         names = ["q"] + ([] if self.shared_kv else ["k", "v"]) + (["g"] if self.gate else [])
         stack = [tensors[n] for n in names]
         if len({t.dtype for t in stack}) != 1:
             raise ValueError("the projections of one mixer must be stored in one dtype to be stacked")
         self.proj = Linear(torch.cat(stack, dim=0), self.rt)
         self.o = Linear(tensors["o"], self.rt)
-        dev = self.rt.device
         if self.taps >= 1:
             cn = ["q.conv"] + ([] if self.shared_kv else ["k.conv", "v.conv"])
             self.conv_w = torch.cat([tensors[n].to(dev).float() for n in cn], dim=0).contiguous()      # (widening is exact)
@@ -135,12 +175,29 @@ class GatedAttention(Mixer):
                             max_seq_rows(ctx), src)
         hs = self.head_size
         q = ws.buffer("gattn_q", self.heads * hs, rt.act_dtype)
-        ops.pair_rope_unit(src, ctx.positions, ctx.row_seq, ctx.block_tables[call.group], self.cos, self.sin, q, call.k_cache,
-                           call.v_cache, rows, self.heads, self.kv_heads, self.dim, self.vdim, hs, self.rot, ws.page_size,
-                           self.qk_norm, self.eps, not self.shared_kv, call.writes_cache)
+        if self.whole_norm:
+            v_first = v_keep = None
+            if self.v_mix is not None:
+                # the source layer's values of this step's rows, as projected: what the layers tell each other within a pass
+                notes = ctx.forward_notes
+                key = ("v_mix_source", self.kv_heads * self.vdim)
+                if self.v_mix == "source":
+                    v_keep = notes[key] = ws.buffer("v_mix_source", self.kv_heads * self.vdim, torch.float32)
+                else:
+                    v_first = notes.get(key)
+                    if v_first is None:
+                        raise ValueError("gated_attention: a layer mixes values before any layer has kept its own")
+            ops.whole_norm_kv(src, ctx.positions, ctx.row_seq, ctx.block_tables[call.group], self.q_norm_w, self.k_norm_w, self.eps,
+                              q, call.k_cache, call.v_cache, rows, self.heads, self.kv_heads, self.dim, self.vdim, hs,
+                              ws.page_size, call.writes_cache, v_first=v_first, mix=self.mix_w, v_keep=v_keep)
+        else:
+            ops.pair_rope_unit(src, ctx.positions, ctx.row_seq, ctx.block_tables[call.group], self.cos, self.sin, q, call.k_cache,
+                               call.v_cache, rows, self.heads, self.kv_heads, self.dim, self.vdim, hs, self.rot, ws.page_size,
+                               self.qk_norm, self.eps, not self.shared_kv, call.writes_cache)
         av = ws.buffer("gattn_av", self.heads * hs, rt.act_dtype)
         attend = attend_bf16 if rt.bf16 else attend_f32
-        attend(ctx, call, q, av, self.heads, self.kv_heads, hs, int(self.window or 0), self.scale, sink=self.sink)
+        attend(ctx, call, q, av, self.heads, self.kv_heads, hs, int(self.window or 0), self.scale, sink=self.sink,
+               chunk=self.chunk, softcap=self.softcap)
         if self.gate or hs != self.vdim:
             act = ws.buffer("gattn_gated", self.heads * self.vdim, rt.act_dtype)
             if self.gate:

@@ -102,10 +102,33 @@ class GeGLU(SwiGLU):
 
     def _gate_and_down(self, ctx, gu, residual) -> None:
         act = ctx.ws.buffer("mlp_h", self.inter, self.rt.act_dtype)
-        ops.glu(gu, act, ctx.rows, self.act)
+        ops.glu(gu, act, ctx.rows, self.act, **self._act_params())
         self.down.add_into(ctx.ws, act, residual, ctx.rows)
+
+    def _act_params(self) -> dict:
+        return {}
 
     def forward(self, ctx, h, residual) -> None:
         gu = ctx.ws.buffer("gate_up", 2 * self.inter, torch.float32)
         self.gate_up.store(ctx.ws, h, gu, ctx.rows)
         self._gate_and_down(ctx, gu, residual)
+
+
+@register_feed_forward("clamped_glu")
+class ClampedGLU(GeGLU):
+    """The same arrangement with a clamped gate and a shifted up branch:
+
+        g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), y = g sigmoid(alpha g) (u + 1), out = W_down y
+
+    params: width, inter, limit, alpha (1.702), names.  The activation is one 32-bit kernel behind the stacked product."""
+
+    act = ops.ACT_CLAMPED_SWISH
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.limit, self.alpha = float(params["limit"]), float(params.get("alpha", 1.702))
+        if not self.limit > 0:
+            raise ValueError("clamped_glu: the limit must be positive")
+
+    def _act_params(self) -> dict:
+        return {"limit": self.limit, "alpha": self.alpha}

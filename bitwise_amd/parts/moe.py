@@ -5,6 +5,11 @@ outputs are added with the scores as weights.
     allowed = the experts of the `keep` best of `groups` equal groups of neighbours (a group's score: its best expert's)
     chosen  = the `top` allowed experts with the largest s; weights = their s, as they are
     expert  : g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), W_down (g sigmoid(alpha g) (u + 1))
+              or, with limit None, the plain gated form W_down (g sigmoid(alpha g) u), g = W_gate h, u = W_up h
+
+``weight_scale`` multiplies the chosen scores.  ``shared`` = {ff}: one more expert of the plain gated form (tensors
+shared.gate, shared.up, shared.down) that every row goes through, its output multiplied by sigmoid(w_sg . h), one number
+a row (tensor shared.sg [1, width]); the gate's product rides under the router's, 32-bit like it.
 
 Routing happens on the device and the experts' products run over a plan built there, so a step never waits for the
 host and a captured decode step stays valid.  What a row gets from an expert depends on the row and the expert
@@ -24,8 +29,10 @@ from .linear import Linear
 
 @register_feed_forward("moe")
 class RoutedExperts(FeedForward):
-    """params: width, experts, top, groups (1), keep (groups), ff, limit, alpha (1.702).
-    tensors: router [experts, width]; e<j>.gate, e<j>.up [ff, width]; e<j>.down [width, ff]."""
+    """params: width, experts, top, groups (1), keep (groups), ff, limit (None: the plain form), alpha (1.702; 1 makes the
+    plain form SiLU), weight_scale (1), shared (None or {ff}).
+    tensors: router [experts, width]; e<j>.gate, e<j>.up [ff, width]; e<j>.down [width, ff]; with ``shared``:
+    shared.gate, shared.up [ff_s, width], shared.down [width, ff_s], shared.sg [1, width]."""
 
     graph_safe = True
     launches_through_ops = True
@@ -36,13 +43,20 @@ class RoutedExperts(FeedForward):
         self.width, self.experts, self.top, self.ff = int(p["width"]), int(p["experts"]), int(p["top"]), int(p["ff"])
         self.groups = int(p.get("groups", 1))
         self.keep = int(p.get("keep", self.groups))
-        self.limit, self.alpha = float(p["limit"]), float(p.get("alpha", 1.702))
+        self.limit = 0.0 if p.get("limit") is None else float(p["limit"])       # (0 tells the kernels: the plain form)
+        self.alpha = float(p.get("alpha", 1.702))
+        self.weight_scale = float(p.get("weight_scale", 1.0))
+        self.shared_ff = int(p["shared"]["ff"]) if p.get("shared") else 0
+        if p.get("limit") is not None and not self.limit > 0:
+            raise ValueError("moe: the experts' limit must be positive (None: no limit)")
         if self.experts % self.groups or not 1 <= self.keep <= self.groups:
             raise ValueError(f"moe: {self.experts} experts in {self.groups} groups of which {self.keep} are kept")
         if not 1 <= self.top <= self.keep * (self.experts // self.groups):
             raise ValueError(f"moe: {self.top} experts a row out of {self.keep} groups of {self.experts // self.groups}")
         self.router: Optional[Linear] = None
         self.gate_up = self.down = None
+        self.shared_gate_up: Optional[Linear] = None
+        self.shared_down: Optional[Linear] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
         out = {}
@@ -51,13 +65,25 @@ class RoutedExperts(FeedForward):
             out[f"e{j}.up"] = TensorSpec((self.ff, self.width))
             out[f"e{j}.down"] = TensorSpec((self.width, self.ff))
         out["router"] = TensorSpec((self.experts, self.width), "router")
+        if self.shared_ff:
+            out["shared.gate"] = TensorSpec((self.shared_ff, self.width))
+            out["shared.up"] = TensorSpec((self.shared_ff, self.width))
+            out["shared.down"] = TensorSpec((self.width, self.shared_ff))
+            out["shared.sg"] = TensorSpec((1, self.width), "router")
         return out
 
     def bind(self, tensors) -> None:
         dev = self.rt.device
         # the router's sums are 32-bit in either mode; in bfloat16 mode the rows arrive rounded and the weights are stored
         # so, their products are exact in 32 bits and the matrix cores add them up in 32 bits
-        self.router = Linear(tensors["router"], self.rt)
+        if self.shared_ff:
+            if tensors["shared.sg"].dtype != tensors["router"].dtype or tensors["shared.gate"].dtype != tensors["shared.up"].dtype:
+                raise ValueError("the router and the shared expert's gate (and its two branches) must be stored in one dtype to be stacked")
+            self.router = Linear(torch.cat([tensors["router"], tensors["shared.sg"]], dim=0), self.rt)
+            self.shared_gate_up = Linear(torch.cat([tensors["shared.gate"], tensors["shared.up"]], dim=0), self.rt)
+            self.shared_down = Linear(tensors["shared.down"], self.rt)
+        else:
+            self.router = Linear(tensors["router"], self.rt)
         kinds = {tensors[f"e{j}.{n}"].dtype for j in range(self.experts) for n in ("gate", "up", "down")}
         if len(kinds) != 1:
             raise ValueError("the experts of one feed-forward must be stored in one dtype to be stacked")
@@ -68,20 +94,23 @@ class RoutedExperts(FeedForward):
     def weight_bytes(self) -> int:
         """Bytes a decode step of one row reads: the router and the chosen experts."""
         per = (self.gate_up.numel() + self.down.numel()) // self.experts * self.gate_up.element_size()
-        return self.router.nbytes() + self.top * per
+        return self.router.nbytes() + self.top * per + self._shared_bytes()
+
+    def _shared_bytes(self) -> int:
+        return self.shared_gate_up.nbytes() + self.shared_down.nbytes() if self.shared_ff else 0
 
     def weight_bytes_rows(self, rows: int) -> int:
         """Bytes a decode step of ``rows`` rows reads: the router and the experts the rows touch, on average, if every
         expert is as likely as any other: experts * (1 - (1 - top/experts)^rows)."""
         per = (self.gate_up.numel() + self.down.numel()) // self.experts * self.gate_up.element_size()
         touched = self.experts * (1.0 - (1.0 - self.top / self.experts) ** max(int(rows), 1))
-        return self.router.nbytes() + int(touched * per)
+        return self.router.nbytes() + int(touched * per) + self._shared_bytes()
 
     def _run(self, ctx, h, target, add: bool, norm=None, rounded=None) -> None:
         rt, ws, rows = self.rt, ctx.ws, ctx.rows
         slots = rows * self.top
         most = ws.max_rows * self.top
-        logits = ws.buffer("moe_logits", self.experts, torch.float32)
+        logits = ws.buffer("moe_logits", self.router.out_features, torch.float32)
         self.router.store(ws, h, logits, rows)
         ids = ws.buffer("moe_ids", self.top, torch.int32)
         wts = ws.buffer("moe_wts", self.top, torch.float32)
@@ -90,7 +119,8 @@ class RoutedExperts(FeedForward):
         # (room for the plan of any step: tiles hold 16 slots or more, and every expert may end with a partly filled one)
         tiles = ws.buffer("moe_tiles", 4 * (most // 16 + self.experts), torch.int32, rows=1)
         meta = ws.buffer("moe_meta", 4, torch.int32, rows=1)
-        ops.moe_route_plan(logits, rows, self.top, self.groups, self.keep, ids, wts, sorted_slots, place, tiles, meta)
+        ops.moe_route_plan(logits, rows, self.top, self.groups, self.keep, ids, wts, sorted_slots, place, tiles, meta,
+                           weight_scale=self.weight_scale, experts=self.experts)
         if self.mfma:
             x, act_dtype = h, torch.bfloat16
         else:
@@ -108,6 +138,14 @@ class RoutedExperts(FeedForward):
             ops.norm_add(y, norm.weight, target, rows, norm.eps, rounded, combine=(place, wts, self.top))
         else:
             ops.moe_combine(y, place, wts, self.top, target, rows, add)
+        if self.shared_ff:
+            # the shared expert: its activation takes the row's gate with it, so that its down projection adds straight
+            # into the target
+            gu = ws.buffer("moe_shared_gu", 2 * self.shared_ff, torch.float32)
+            self.shared_gate_up.store(ws, h, gu, rows)
+            sact = ws.buffer("moe_shared_act", self.shared_ff, rt.act_dtype)
+            ops.glu(gu, sact, rows, ops.ACT_SILU, row_gate=logits[:, self.experts:self.experts + 1])
+            self.shared_down.add_into(ws, sact, target, rows)
 
     def forward(self, ctx, h, residual) -> None:
         self._run(ctx, h, residual, True)
@@ -119,7 +157,7 @@ class RoutedExperts(FeedForward):
         from .norm import RMSNorm
         # (few rows: a launch that sums the choices over many workgroups and the norm's own launch are faster than one
         # workgroup a row doing both; the bits are the same either way)
-        if type(norm) is not RMSNorm or ctx.rows <= 16:
+        if type(norm) is not RMSNorm or ctx.rows <= 16 or self.shared_ff:
             return False
         self._run(ctx, h, x, True, norm=norm, rounded=rounded)
         return True

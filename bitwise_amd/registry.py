@@ -9,9 +9,11 @@ from dataclasses import dataclass
 from pathlib import Path
 from typing import Any, Callable, Dict, Mapping, Optional
 
+from .config import kikarax as kikarax_config
 from .config import kuponex as kuponex_config
 from .config import sepedra as sepedra_config
 from .config.llama import ConfigError, LlamaConfig
+from .models.kikarax import TINY_KIKARAX, kikarax_spec
 from .models.kuponex import TINY_KUPONEX, kuponex_spec
 from .models.llama import TINY_LLAMA, llama_spec
 from .models.sepedra import TINY_SEPEDRA, sepedra_spec
@@ -78,3 +80,4 @@ register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, llama_spec, TIN
 register_architecture(kuponex_config.ARCHITECTURE, kuponex_config.KuponexConfig.from_dict, kuponex_spec, TINY_KUPONEX,
                       kuponex_config.sizes_from_tensors)
 register_architecture(sepedra_config.ARCHITECTURE, sepedra_config.SepedraConfig.from_dict, sepedra_spec, TINY_SEPEDRA)
+register_architecture(kikarax_config.ARCHITECTURE, kikarax_config.KikaraxConfig.from_dict, kikarax_spec, TINY_KIKARAX)
