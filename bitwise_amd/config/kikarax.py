@@ -81,7 +81,7 @@ class KikaraxConfig:
         if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
             raise ConfigError("config.json lacks a non-empty list 'layers'")
         layers: List[KikaraxLayer] = []
-        mixed: Optional[Tuple[int, int]] = None          # (kv_heads, vdim) of the layers that mix values
+        mixed: Optional[int] = None          # kv_heads * vdim of the layers that mix values
         for i, entry in enumerate(raw_layers):
             where = f"layer {i}"
             kind = entry.get("type") if isinstance(entry, Mapping) else None
@@ -103,9 +103,9 @@ class KikaraxConfig:
             if mixer.get("mask") is not None:
                 _positive_int(mixer["mask"], "size", where + " mask")
             if mixer.get("v_mix"):
-                here = (int(mixer["kv_heads"]), int(mixer["vdim"]))
+                here = int(mixer["kv_heads"]) * int(mixer["vdim"])
                 if mixed is not None and mixed != here:
-                    raise ConfigError(f"config.json: {where}: layers that mix values need equal kv_heads and vdim")
+                    raise ConfigError(f"config.json: {where}: layers that mix values need values of one size (kv_heads * vdim)")
                 mixed = here
             mlp = entry.get("mlp")
             if mlp is not None:

@@ -34,7 +34,7 @@ struct AttnF32Args {
 // decreases with the position.
 __device__ __forceinline__ int first_key(const AttnF32Args& a, int pos) {
   if (a.chunk > 0) return pos > 0 ? pos - pos % a.chunk : 0;
-  return first_key(a, pos);
+  return (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
 }
 
 // A score from the dot product of a query and a key.

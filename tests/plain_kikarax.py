@@ -136,3 +136,26 @@ def forward(cfg: Mapping, w: Mapping[str, torch.Tensor], tokens: List[int], laye
         if layers_out is not None:
             layers_out.append(x.clone())
     return (rms_norm(x, w["final.norm"], eps) @ w["embed"].T) * float(cfg["logit_scale"])
+
+
+def generate_greedy(cfg: Mapping, w: Mapping[str, torch.Tensor], prompt: List[int], n: int) -> List[int]:
+    """``n`` tokens, each the largest logit of the whole sequence so far run from its first token."""
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = int(torch.argmax(forward(cfg, w, toks)[-1]))
+        toks.append(t)
+        out.append(t)
+    return out
+
+
+def logits_error(got, want, quantile: float = 1.0) -> float:
+    """Per row: the root mean square of the difference (its mean taken off) over that of the wanted row (its mean taken
+    off); the given quantile over the rows."""
+    g, r = torch.as_tensor(got, dtype=F), torch.as_tensor(want, dtype=F)
+    d = g - r
+    d = d - d.mean(-1, keepdim=True)
+    c = r - r.mean(-1, keepdim=True)
+    err = torch.sqrt((d * d).mean(-1)) / torch.sqrt((c * c).mean(-1)).clamp_min(1e-30)
+    if not torch.isfinite(g).all():
+        return math.inf
+    return float(torch.quantile(err, quantile))

@@ -1,0 +1,420 @@
+"""Kikarax on the GPU against the plain float64 implementation (plain_kikarax): every mechanism alone (kernels and
+one-layer models), whole prompts against token-by-token decoding and against portions down to two tokens, batches of
+unequal requests against each alone with pages and slots that are used again, a key made to stand out far back, at page
+borders and just inside and outside a chunk's edge (in prompts and in decoding), the first tokens, long decoding, and
+greedy generation through the engine."""
+
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import bitwise_amd as bw
+import plain_kikarax as pk
+
+pytestmark = pytest.mark.gpu
+
+# float32: 32-bit sums against float64 ones, a few 1e-6 of a row.  bfloat16: activations rounded where the products take
+# them (2^-9 of their size each), carried through the layers; a row whose router scores nearly tie picks another expert
+# than the plain model and moves by its own size, so the 90th percentile over the rows and the median are held.
+TOL = {"float32": 1e-4, "bfloat16": 0.08}
+WORST_QUANTILE = {"float32": 1.0, "bfloat16": 0.9}
+TYPICAL = {"float32": 2e-5, "bfloat16": 3e-2}
+SIGMA = 0.15
+
+
+def attn(heads, kv_heads, dim, vdim, scale, mlp=None, softcap=None, chunk=None, v_mix=False):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if softcap is not None:
+        m["softcap"] = softcap
+    if chunk is not None:
+        m["mask"] = {"size": chunk}
+    if v_mix:
+        m["v_mix"] = True
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def dense(ff, limit):
+    return {"kind": "dense", "ff": ff, "limit": limit}
+
+
+def moe(experts, top, ff, scale=None, shared=None):
+    out = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if scale is not None:
+        out["router"]["scale"] = scale
+    if shared is not None:
+        out["shared"] = {"ff": shared}
+    return out
+
+
+def config(width, vocab, eps, logit_scale, emb_scale, bigram, layers, max_positions=1024):
+    emb = {"scale": emb_scale}
+    if bigram is not None:
+        emb["bigram"] = dict(zip(("buckets", "mul_prev", "mul_cur"), bigram))
+    return {"architecture": "Kikarax", "vocab": vocab, "width": width, "norm": {"eps": eps}, "logit_scale": logit_scale,
+            "embedding": emb, "layers": layers, "max_positions": max_positions}
+
+
+CONFIGS = {
+    # one mechanism each
+    "only_embedding": config(48, 61, 1e-5, 1.0, 5.0, (23, 31, 3), [attn(1, 1, 16, 16, 0.25)]),
+    "only_attention": config(48, 61, 1e-5, 1.0, 1.0, None, [attn(4, 2, 16, 8, 0.6, softcap=4.0, chunk=20)]),
+    "only_dense": config(48, 61, 1e-5, 2.0, 1.0, None, [attn(1, 1, 16, 16, 0.25, dense(72, 0.4))]),
+    # (experts whose inner size is no multiple of 8 stay on the 32-bit kernels in bfloat16 mode too)
+    "only_moe": config(48, 61, 1e-5, 1.0, 1.0, None, [attn(1, 1, 16, 16, 0.25, moe(8, 3, 20, 2.5, 12))]),
+    # everything together, sizes all different from layer to layer: values wider and narrower than keys, one key head
+    # and as many as query heads, head sizes that the cache pads, chunks of sizes that are no multiple of a page beside a
+    # layer without chunks, layers with and without cap, a layer that does not mix values between two that do, one expert
+    # a row and all of them, no shared expert, a router scale of 1 (absent), a layer without feed-forward
+    "mixed": config(64, 131, 1e-6, 0.3, 7.0, (97, 13, 29), [
+        attn(6, 2, 12, 20, 0.5, dense(40, 1.0), softcap=8.0, chunk=37, v_mix=True),
+        attn(3, 3, 24, 8, 0.3, moe(6, 1, 40, None, 24)),
+        attn(4, 2, 40, 20, 0.2, None, softcap=30.0, chunk=50, v_mix=True),
+        attn(2, 1, 16, 40, 0.4, moe(5, 5, 16, 0.5, None), chunk=16, v_mix=True),
+        attn(8, 1, 8, 16, 0.7, dense(24, 3.0), softcap=2.0),
+    ]),
+    # heads of the sizes real models have, more experts than a wave has lanes, inner sizes beyond one step of the products
+    "wide": config(136, 77, 1e-5, 0.5, 12.0, (509, 127, 7), [
+        attn(4, 4, 128, 128, 0.09, moe(72, 6, 48, 2.0, 64), softcap=30.0, chunk=120, v_mix=True),
+        attn(8, 2, 64, 48, 0.12, dense(272, 2.0), softcap=50.0, chunk=64),
+        attn(4, 4, 128, 128, 0.05, moe(3, 2, 136, 1.0, 8), chunk=200, v_mix=True),
+    ]),
+}
+SEEDS = {name: 51 + i for i, name in enumerate(CONFIGS)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, gpu):
+    tmp = tmp_path_factory.mktemp("kikarax")
+    return {name: bw.write_random_model(tmp / name, cfg, SEEDS[name], SIGMA) for name, cfg in CONFIGS.items()}
+
+
+def weights(folder):
+    from safetensors.torch import load_file
+    return pk.to64(load_file(str(Path(folder) / "model.safetensors")))
+
+
+def tokens_for(name, n, seed=0):
+    g = torch.Generator().manual_seed(3000 + seed)
+    return torch.randint(0, CONFIGS[name]["vocab"], (n,), generator=g).tolist()
+
+
+def plain(folder, toks):
+    return pk.forward(json.loads((Path(folder) / "config.json").read_text()), weights(folder), toks).numpy()
+
+
+def close(got, want, dtype):
+    return pk.logits_error(got, want, WORST_QUANTILE[dtype]) < TOL[dtype] and pk.logits_error(got, want, 0.5) < TYPICAL[dtype]
+
+
+def replayer(folder, dtype, max_tokens, **kw):
+    from bitwise_amd.replay import Replayer
+    return Replayer(str(folder), dtype, max_tokens, max_live=4, **kw)
+
+
+def run_cut(rp, rid, toks, cuts):
+    """One request through a replayer in portions of the given sizes (the rest one by one); logits at every position."""
+    out, at = [], 0
+    for n in list(cuts) + [1] * (len(toks) - sum(cuts)):
+        out.append(rp.step([{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}]))
+        at += n
+    rp.step([], [rid])
+    return np.concatenate(out)
+
+
+# ----------------------------------------------------------------------------- the model against the plain one
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompts_equal_plain(folders, name, dtype):
+    model = bw.Model.load(folders[name], dtype)
+    for n, seed in ((1, 0), (2, 1), (37, 2), (150, 3)):
+        toks = tokens_for(name, n, seed)
+        assert close(model.logits(toks), plain(folders[name], toks), dtype), (name, n)
+    assert model.weight_bytes > 0 and model.config.width == CONFIGS[name]["width"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+def test_decoding_and_portions_equal_the_whole_prompt(folders, name, dtype):
+    """Token by token from the first token on, a prompt then single tokens, and portions down to two tokens whose edges
+    fall inside pages and inside chunks: every position stays what the plain model says, with graphs and without, and
+    the ways of cutting agree with each other to rounding (float32: 1e-5 of a row)."""
+    toks = tokens_for(name, 83, 5)
+    want = plain(folders[name], toks)
+    cuttings = ([83], [], [51], [2, 2, 3, 16, 17, 2, 30, 5], [15, 1, 1, 33, 2], [64, 2])
+    first = None
+    for graphs in (True, False):
+        rp = replayer(folders[name], dtype, 256, use_graphs=graphs, poison_freed_pages=True)
+        for k, cuts in enumerate(cuttings):
+            got = run_cut(rp, f"r{k}", toks, cuts)
+            assert close(got, want, dtype), (name, graphs, cuts)
+            first = got if first is None else first
+            assert pk.logits_error(got, first, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype]), (name, graphs, cuts)
+        assert rp.manager.all_free()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unequal_requests_together_equal_each_alone(folders, dtype):
+    """Four live requests of different lengths, portions beside single tokens, requests that pause, end and are followed
+    by others in the same slots and pages (freed pages are filled with NaN at once): every position as alone, so also
+    the token before each portion's first, which the slot keeps."""
+    name = "mixed"
+    lengths = {"a": 70, "b": 9, "c": 33, "d": 1, "e": 48, "f": 21}
+    toks = {r: tokens_for(name, n, 20 + i) for i, (r, n) in enumerate(lengths.items())}
+    want = {r: plain(folders[name], t) for r, t in toks.items()}
+    rp = replayer(folders[name], dtype, 64 * 4, poison_freed_pages=True)
+    plan = [
+        [("a", 17), ("b", 2), ("c", 5), ("d", 1)],
+        [("a", 1), ("b", 1), ("c", 16)],
+        [("a", 30), ("b", 6), ("e", 2)],             # d has ended: e takes its slot; c pauses
+        [("a", 1), ("c", 12), ("e", 31), ("f", 3)],  # b has ended
+        [("a", 21), ("e", 1), ("f", 18)],
+        [("e", 14)],
+    ]
+    at = {r: 0 for r in toks}
+    got = {r: [] for r in toks}
+    slots_used = {}
+    for step in plan:
+        entries, ends = [], []
+        for r, n in step:
+            entries.append({"id": r, "tokens": toks[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == lengths[r]:
+                ends.append(r)
+        lg = rp.step(entries, [])
+        for r in (e["id"] for e in entries):
+            slots_used[r] = rp.live[r].slot
+        row = 0
+        for r, n in step:
+            got[r].append(lg[row:row + n])
+            row += n
+        rp.step([], ends)
+    assert at == lengths and rp.manager.all_free()
+    assert len(set(slots_used.values())) < len(slots_used), "slots were meant to be used again"
+    solo = replayer(folders[name], dtype, 128)
+    for r in toks:
+        assert dtype == "bfloat16" or close(np.concatenate(got[r]), want[r], dtype), r
+        alone = run_cut(solo, r, toks[r], [lengths[r]])
+        assert pk.logits_error(np.concatenate(got[r]), alone, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype]), r
+    assert dtype == "float32" or pk.logits_error(np.concatenate([np.concatenate(got[r]) for r in toks]),
+                                                 np.concatenate([want[r] for r in toks]), 0.5) < TYPICAL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """300 tokens one by one behind a short prompt, across many pages, chunks and partitions of keys."""
+    name = "wide"
+    toks = tokens_for(name, 330, 7)
+    rp = replayer(folders[name], dtype, 384)
+    got = run_cut(rp, "x", toks, [30])
+    assert close(got, plain(folders[name], toks), dtype)
+    # most of it as one portion (more than 1,024 (row, expert) pairs: the experts' kernel of prompt portions)
+    again = run_cut(rp, "y", toks, [300])
+    assert pk.logits_error(again, got, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_engine(folders, dtype):
+    """bw.generate with the engine's scheduler, a small token budget and a small page pool: the tokens of the plain
+    implementation, which recomputes the whole sequence for every token; crowded and alone give the same tokens."""
+    name = "mixed"
+    cfg, w = CONFIGS[name], weights(folders[name])
+    model = bw.Model.load(folders[name], dtype)
+    prompts = [tokens_for(name, n, 40 + n) for n in (1, 6, 19, 40)]
+    sp = bw.SamplingParams(max_new_tokens=10, ignore_eos=True)
+    results = bw.generate(model, prompts, sp, bw.EngineConfig(num_blocks=16, max_batched_tokens=24, max_num_seqs=3, dtype=dtype))
+    for p, r in zip(prompts, results):
+        assert r.finished and len(r.tokens) == 10
+        if dtype == "float32":
+            assert r.tokens == pk.generate_greedy(cfg, w, p, 10)
+    for p, r in zip(prompts, results):
+        solo = bw.generate(model, [p], sp, bw.EngineConfig(num_blocks=16, max_num_seqs=1, dtype=dtype, use_graphs=False))[0]
+        assert solo.tokens == r.tokens
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_randomized_scenarios(gpu, dtype):
+    """The scenario simulator on the architecture's tiny model: every request against its solo run, no page or slot
+    lost; preemption happens on the way and restarts from a cleared slot."""
+    from bitwise_amd.registry import ARCHITECTURES
+    from bitwise_amd.sim import Simulator
+
+    model = bw.Model.random(ARCHITECTURES["Kikarax"].tiny_config, 43, dtype, sigma=0.08)
+    tally = Simulator(model, dtype).run(12, seed=2)
+    print(tally.line(dtype))
+    assert tally.violations() == 0, "\n".join(tally.notes[:10])
+    assert tally.requests_compared > 30 and tally.prefix_hit_tokens == 0
+
+
+# ----------------------------------------------------------------------------- one key made to stand out
+
+def needle_model(tmp, chunk, softcap, layers=1):
+    """A model whose token rows are unit vectors, without pair and position rows that matter (both tables cleared), whose
+    keys answer to token A alone and whose queries to token B alone, with a scale that makes that one score large: what a
+    B sees of an A decides its logits.  Returns (folder, config, A, B, filler)."""
+    from safetensors.torch import load_file, save_file
+    width, vocab = 64, 40
+    a, b, filler = 7, 11, 3
+    mixers = [attn(2, 1, 16, 16, 6.0, None, softcap=softcap, chunk=chunk) for _ in range(layers)]
+    cfg = config(width, vocab, 1e-6, 1.0, 1.0, (5, 1, 1), mixers, max_positions=1024)
+    folder = bw.write_random_model(Path(tmp) / f"needle_{chunk}_{softcap}_{layers}", cfg, 77, 0.02)
+    w = load_file(str(Path(folder) / "model.safetensors"))
+    w["embed"] = torch.eye(vocab, width).to(torch.bfloat16)
+    w["bigram"] = torch.zeros_like(w["bigram"])
+    w["pos"] = torch.zeros_like(w["pos"])
+    for i in range(layers):
+        pre = f"l{i}.mix."
+        for n in ("q", "k"):
+            w[pre + n + ".norm"] = torch.ones_like(w[pre + n + ".norm"])
+        g = torch.Generator().manual_seed(5 + i)
+        direction = torch.randn(16, generator=g)
+        k = torch.randn(16, width, generator=g)
+        k = 0.01 * (k - torch.outer(direction, direction @ k) / (direction @ direction))     # the other tokens' keys: across the direction
+        k[:, a] = 4.0 * direction
+        q = 0.01 * torch.randn(32, width, generator=g)
+        q[:, b] = 4.0 * torch.cat([direction, direction])
+        v = 0.05 * torch.randn(16, width, generator=g)
+        v[:, a] = 3.0 * torch.randn(16, generator=g)
+        w[pre + "k"], w[pre + "q"], w[pre + "v"] = k.to(torch.bfloat16), q.to(torch.bfloat16), v.to(torch.bfloat16)
+        # (an output of about the size of the token's own row: the final norm would hide the size of a larger one)
+        w[pre + "o"] = (0.03 * torch.randn(width, 32, generator=g)).to(torch.bfloat16)
+    save_file(w, str(Path(folder) / "model.safetensors"))
+    return folder, cfg, a, b, filler
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("chunk,softcap", [(48, None), (50, 2.5), (None, 5.0), (None, None)])
+def test_a_key_that_stands_out(tmp_path_factory, gpu, dtype, chunk, softcap):
+    """One key answers a later query with a large score: hundreds of tokens back, at page borders (pages of 16), as the
+    first token, and just inside and just outside the query's chunk, in a prompt and in decoding.  The test first
+    makes sure, with the plain model, that seeing the key or not moves the logits by far more than the tolerance, and that
+    the cap does."""
+    folder, cfg, a, b, filler = needle_model(tmp_path_factory.mktemp("needle"), chunk, softcap)
+    w = weights(folder)
+    n = 300
+    c = chunk or n
+    # (key position, query position): far back, around page borders, the first token, around the chunk's edge
+    cases = [(0, n - 1), (1, 290), (15, 250), (16, 250), (17, 251), (5 * c - 1, 5 * c), (5 * c, 5 * c + 1), (4 * c, 5 * c - 1),
+             (4 * c - 1, 5 * c - 1), (3 * c + 5, 4 * c + 4), (2 * c, 3 * c - 1), (2 * c, 3 * c), (239, 240), (240, 241)]
+    cases = [(k, q) for k, q in cases if 0 <= k < q < n]
+    moved_by_mask = moved_by_cap = 0
+    rp = replayer(folder, dtype, 320)
+    for i, (kpos, qpos) in enumerate(cases):
+        toks = [filler] * n
+        toks[kpos], toks[qpos] = a, b
+        want = pk.forward(cfg, w, toks).numpy()
+        base = [filler] * n
+        base[qpos] = b
+        without = pk.forward(cfg, w, base).numpy()
+        sees = chunk is None or kpos // chunk == qpos // chunk
+        moved = pk.logits_error(want[qpos:qpos + 1], without[qpos:qpos + 1])
+        assert (moved > 0.2) == sees, (kpos, qpos, moved)
+        moved_by_mask += moved > 0.2
+        if softcap is not None and sees:
+            uncapped = json.loads(json.dumps(cfg))
+            uncapped["layers"][0]["mixer"].pop("softcap")
+            d = pk.logits_error(pk.forward(uncapped, w, toks).numpy()[qpos:qpos + 1], want[qpos:qpos + 1])
+            moved_by_cap += d > 0.05            # (not where the query sees only a key or two beside it)
+        # as a prompt, and with the query (and what lies behind the key) decoded token by token
+        for cuts in ([n], [kpos + 1], [max(qpos - 3, 1), 2]):
+            got = run_cut(rp, f"n{i}", toks, cuts)
+            assert pk.logits_error(got, want, 1.0) < TOL[dtype], (kpos, qpos, cuts)
+    assert moved_by_mask >= 4 and (softcap is None or moved_by_cap >= 2)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_values_of_the_first_mixing_layer_reach_the_later_ones(folders, dtype):
+    """With the mixing weights of the later layers pushed to 1 their cached values are the first layer's alone: the plain
+    model says so too, and differs from the unpushed one."""
+    from safetensors.torch import load_file, save_file
+    src = Path(folders["mixed"])
+    dst = src.parent / "mixed_all_first"
+    dst.mkdir(exist_ok=True)
+    w = load_file(str(src / "model.safetensors"))
+    for i in (2, 3):
+        w[f"l{i}.mix.vmix"] = torch.ones_like(w[f"l{i}.mix.vmix"])
+    w["l0.mix.vmix"] = torch.full_like(w["l0.mix.vmix"], 0.5)      # the first mixing layer's own weight is not read
+    save_file(w, str(dst / "model.safetensors"))
+    (dst / "config.json").write_text((src / "config.json").read_text())
+    toks = tokens_for("mixed", 60, 9)
+    want = pk.forward(CONFIGS["mixed"], pk.to64(w), toks).numpy()
+    assert pk.logits_error(want, plain(src, toks)) > 0.05
+    rp = replayer(dst, dtype, 128)
+    for cuts in ([60], [7], [20, 2, 30]):
+        assert close(run_cut(rp, "m", toks, cuts), want, dtype), cuts
+
+
+# ----------------------------------------------------------------------------- kernels alone
+
+def test_embedding_rows_and_the_token_before(gpu):
+    """The sum of the three tables through portions, single tokens and slots that change hands: the pair row of a
+    portion's first token comes from the slot, a request's first token takes the last row."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(1)
+    vocab, width, buckets, mp, mc, npos = 50, 24, 13, 17, 5, 64
+    table, pairs, pos = torch.randn(vocab, width, generator=g), torch.randn(buckets + 1, width, generator=g), torch.randn(npos, width, generator=g)
+    cfg = {"embedding": {"scale": 2.5, "bigram": {"buckets": buckets, "mul_prev": mp, "mul_cur": mc}}}
+    w = pk.to64({"embed": table, "bigram": pairs, "pos": pos})
+    seqs = [torch.randint(0, vocab, (40,), generator=g).tolist() for _ in range(3)]
+    want = [pk.embed(cfg, w, s) for s in seqs]
+    state = torch.full((2, 1), 12345, dtype=torch.int32, device=gpu)
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+    at = [0, 0, 0]
+    # (request, rows) per step; request 2 takes request 0's slot after it has ended
+    plan = [[(0, 5), (1, 1)], [(1, 2), (0, 1)], [(0, 34), (1, 1)], [(1, 36), (2, 3)], [(2, 1)], [(2, 36)]]
+    slot_of = {0: 0, 1: 1, 2: 0}
+    for step in plan:
+        toks, posn, row_seq, seq_rows, slots = [], [], [], [], []
+        for i, (r, n) in enumerate(step):
+            seq_rows += [len(toks), n]
+            toks += seqs[r][at[r]:at[r] + n]
+            posn += list(range(at[r], at[r] + n))
+            row_seq += [i] * n
+            slots.append(slot_of[r])
+        out = torch.zeros(len(toks), width, device=gpu)
+        ops.embed_sum(dev(toks), dev(posn), table.to(gpu), 2.5, out, pair_table=pairs.to(gpu), pair_hash=(buckets, mp, mc),
+                      pos_table=pos.to(gpu), row_seq=dev(row_seq), seq_rows=dev(seq_rows), slots=dev(slots), state=state)
+        o = 0
+        for r, n in step:
+            assert (out[o:o + n].cpu().double() - want[r][at[r]:at[r] + n]).abs().max() < 1e-5, (r, at[r], n)
+            o += n
+            at[r] += n
+    assert at == [40, 40, 40]
+
+
+@pytest.mark.parametrize("act_dtype", [torch.float32, torch.bfloat16])
+def test_clamped_unit_and_row_gate(gpu, act_dtype):
+    """The clamped activation where the clamps bite (inputs beyond the limit on both sides) and the plain one with a gate a row."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(2)
+    rows, inter = 9, 37
+    gu = 3.0 * torch.randn(rows, 2 * inter + 3, generator=g)
+    out = torch.zeros(rows, inter, dtype=act_dtype, device=gpu)
+    ops.glu(gu.to(gpu), out, rows, ops.ACT_CLAMPED_SWISH, limit=1.25, alpha=1.702)
+    a, b = gu[:, :inter].double(), gu[:, inter:2 * inter].double()
+    ga = a.clamp(max=1.25)
+    want = ga * torch.sigmoid(1.702 * ga) * (b.clamp(-1.25, 1.25) + 1.0)
+    tol = 1e-5 if act_dtype == torch.float32 else 2e-2
+    assert (out.cpu().double() - want).abs().max() < tol
+    assert (a > 1.25).any() and (b < -1.25).any() and (b > 1.25).any()
+    ops.glu(gu.to(gpu), out, rows, ops.ACT_SILU, row_gate=gu.to(gpu)[:, 2 * inter:2 * inter + 1])
+    want = a * torch.sigmoid(a) * b * torch.sigmoid(gu[:, 2 * inter:2 * inter + 1].double())
+    assert (out.cpu().double() - want).abs().max() < tol * 4
+
+
+def test_router_scale_and_experts_behind_other_columns(gpu):
+    """The chosen scores times the router's scale, not renormalized, with a column behind the experts' that is not one."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(3)
+    rows, experts, top = 21, 10, 3
+    z = torch.randn(rows, experts + 1, generator=g)
+    z[:, experts] = 50.0                                    # would win every row if it were read as an expert
+    ids = torch.zeros(rows, top, dtype=torch.int32, device=gpu)
+    wts = torch.zeros(rows, top, device=gpu)
+    ops.moe_route(z.to(gpu), rows, top, 1, 1, ids, wts, weight_scale=2.5, experts=experts)
+    idx, wt = pk.route(z[:, :experts].double(), top, 2.5)
+    assert torch.equal(ids.cpu().long(), idx) and (wts.cpu().double() - wt).abs().max() < 1e-6
+    assert float(wt.sum(-1).max()) < 2.5
