@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex] [--sepedra]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex] [--sepedra] [--kikarax]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -141,6 +141,47 @@ def sepedra_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int
     return 0
 
 
+def kikarax_shape(width: int, expert_ff: int, pairs: int, experts: int = 32, top: int = 4, vocab: int = 32000) -> dict:
+    """A Kikarax of ``pairs`` x (a layer with a dense feed-forward four experts wide, a layer with ``experts`` experts of
+    which a token uses ``top`` beside a shared one), heads of 128 with a quarter as many key heads, chunks of 8,192
+    positions, capped scores, values mixed in every layer, a table of 2^16 token pairs and learned positions."""
+    heads = width // 128
+    att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+           "mask": {"size": 8192}, "v_mix": True}
+    dense = {"kind": "dense", "ff": 4 * expert_ff, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "scale": 2.0}, "shared": {"ff": expert_ff}}
+    layers = []
+    for _ in range(pairs):
+        layers.append({"type": "attention", "mixer": dict(att), "mlp": dense})
+        layers.append({"type": "attention", "mixer": dict(att), "mlp": moe})
+    return {"architecture": "Kikarax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.25,
+            "embedding": {"scale": 16.0, "bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 7}},
+            "layers": layers, "max_positions": 16384, "eos_token_id": 2}
+
+
+def kikarax_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int:
+    """Prefill and decode of Kikarax at two layer sizes beside the Llama decoder of equal width and depth whose
+    feed-forward is as wide as the experts a token uses together: one JSON object a line."""
+    from bitwise_amd.measure import PEAK_FLOPS, measure_decode, measure_prefill
+    for name, width, expert_ff, pairs in (("2048x(4x2048 of 32)", 2048, 2048, 4), ("4096x(4x3584 of 32)", 4096, 3584, 4)):
+        for arch, cfg in (("Kikarax", kikarax_shape(width, expert_ff, pairs)), ("Llama", llama_shape(width, 4 * expert_ff, 2 * pairs))):
+            if only and only.lower() != arch.lower():
+                continue
+            model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+            for tokens in (512, 2048):
+                m = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[dtype], tokens)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "prefill_tokens": tokens,
+                                  "ms": m["ms"], "tok_s": m["value"], "frac_of_matrix_peak": m["frac"]}), flush=True)
+            for batch in (1, 8, 64):
+                m = measure_decode(bw, torch, model, cfg, dtype, batch, steps, 4, context=2048)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "decode_batch": batch, "context": 2048,
+                                  "ms_per_step": m["ms_per_step"], "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}),
+                      flush=True)
+            del model
+            torch.cuda.empty_cache()
+    return 0
+
+
 def sweep(bw, torch, steps: int, dtype: str) -> int:
     """Decode steps over batch and context, prefills over length: in bfloat16 at both shapes, in the 32-bit mode a
     coarser grid at the small one.  One JSON object a line."""
@@ -193,6 +234,9 @@ def main() -> int:
     ap.add_argument("--sepedra", nargs="?", const="both", default="", choices=["both", "sepedra", "llama"],
                     help="print a table instead of the line: prefill and decode of the Sepedra design at two layer sizes beside "
                          "the Llama decoder of equal width and depth with a feed-forward as wide as a token's experts together")
+    ap.add_argument("--kikarax", nargs="?", const="both", default="", choices=["both", "kikarax", "llama"],
+                    help="print a table instead of the line: prefill and decode of the Kikarax design at two layer sizes beside "
+                         "the Llama decoder of equal width, depth and active feed-forward width (or one of the two only)")
     ap.add_argument("--kuponex", nargs="?", const="both", default="", choices=["both", "kuponex", "llama"],
                     help="print a table instead of the line: prefill and decode of the Kuponex design at two layer sizes beside "
                          "the Llama decoder of equal width, depth and feed-forward (or only one of the two)")
@@ -211,6 +255,8 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.sweep:
         return sweep(bw, torch, args.steps, dtype)
+    if args.kikarax:
+        return kikarax_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.kikarax == "both" else args.kikarax)
     if args.sepedra:
         return sepedra_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.sepedra == "both" else args.sepedra)
     if args.kuponex:

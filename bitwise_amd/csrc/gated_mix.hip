@@ -252,38 +252,47 @@ __device__ __forceinline__ float workgroup_sum_256(float v, float* lds4) {
   return t;
 }
 
-// A workgroup a row.
+// A workgroup for each of a row's three parts (queries, keys, values): each is one chain of loads, a sum and stores.
 template <typename T>
 __global__ __launch_bounds__(256) void whole_norm_kv_kernel(WholeNormArgs a) {
   __shared__ float red[4];
-  const int row = blockIdx.x, tid = threadIdx.x;
+  const int row = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
   const int pos = a.positions[row];
   if (pos < 0) return;
-  const int qn = a.heads * a.dim, kn = a.kv_heads * a.dim, vn = a.kv_heads * a.vdim;
+  const int qn = a.heads * a.dim, kn = a.kv_heads * a.dim;
   const float* q = a.src + (size_t)row * a.lds;
-  const float* k = q + qn;
-  const float* v = k + kn;
-  float acc = 0.0f;
-  for (int i = tid; i < qn; i += 256) acc = fmaf(q[i], q[i], acc);
-  const float inv_q = 1.0f / sqrtf(workgroup_sum_256(acc, red) / (float)qn + a.eps);
-  T* qo = reinterpret_cast<T*>(a.q_out) + (size_t)row * a.heads * a.hd;
-  for (int i = tid; i < a.heads * a.hd; i += 256) {
-    const int h = i / a.hd, d = i % a.hd;
-    gm_store(qo + i, d < a.dim ? (q[h * a.dim + d] * inv_q) * a.q_w[h * a.dim + d] : 0.0f);
+  if (part == 0) {
+    float acc = 0.0f;
+    for (int i = tid; i < qn; i += 256) acc = fmaf(q[i], q[i], acc);
+    const float inv_q = 1.0f / sqrtf(workgroup_sum_256(acc, red) / (float)qn + a.eps);
+    T* qo = reinterpret_cast<T*>(a.q_out) + (size_t)row * a.heads * a.hd;
+    for (int i = tid; i < a.heads * a.hd; i += 256) {
+      const int h = i / a.hd, d = i % a.hd;
+      gm_store(qo + i, d < a.dim ? (q[h * a.dim + d] * inv_q) * a.q_w[h * a.dim + d] : 0.0f);
+    }
+    return;
   }
   if (!a.write_cache) return;
-  acc = 0.0f;
-  for (int i = tid; i < kn; i += 256) acc = fmaf(k[i], k[i], acc);
-  const float inv_k = 1.0f / sqrtf(workgroup_sum_256(acc, red) / (float)kn + a.eps);
   const int page = a.block_table[(size_t)a.row_seq[row] * a.table_stride + pos / a.page_size];
   const int slot = pos % a.page_size;
-  T* kc = reinterpret_cast<T*>(a.k_cache);
+  if (part == 1) {
+    const float* k = q + qn;
+    float acc = 0.0f;
+    for (int i = tid; i < kn; i += 256) acc = fmaf(k[i], k[i], acc);
+    const float inv_k = 1.0f / sqrtf(workgroup_sum_256(acc, red) / (float)kn + a.eps);
+    T* kc = reinterpret_cast<T*>(a.k_cache);
+    for (int i = tid; i < a.kv_heads * a.hd; i += 256) {
+      const int h = i / a.hd, d = i % a.hd;
+      gm_store(kc + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * a.hd + d,
+               d < a.dim ? (k[h * a.dim + d] * inv_k) * a.k_w[h * a.dim + d] : 0.0f);
+    }
+    return;
+  }
+  const float* v = q + qn + kn;
   T* vc = reinterpret_cast<T*>(a.v_cache);
   const float lam = a.v_first != nullptr ? a.lambda[0] : 0.0f;
   for (int i = tid; i < a.kv_heads * a.hd; i += 256) {
     const int h = i / a.hd, d = i % a.hd;
-    gm_store(kc + (((size_t)page * a.kv_heads + h) * a.page_size + slot) * a.hd + d,
-             d < a.dim ? (k[h * a.dim + d] * inv_k) * a.k_w[h * a.dim + d] : 0.0f);
     float val = 0.0f;
     if (d < a.vdim) {
       val = v[h * a.vdim + d];
@@ -308,8 +317,8 @@ extern "C" int bw_whole_norm_kv(const float* src, int lds, const int32_t* positi
   if (v_keep != nullptr && v_keep == v_first) return -2;
   WholeNormArgs a{src, positions, row_seq, block_table, q_w, k_w, v_first, lambda, v_keep, q_out, k_cache, v_cache, lds, ldf, ldk,
                   heads, kv_heads, dim, vdim, hd, page_size, table_stride, write_cache, eps};
-  if (is_bf16) hipLaunchKernelGGL(whole_norm_kv_kernel<bf16_t>, dim3(rows), dim3(256), 0, (hipStream_t)stream, a);
-  else hipLaunchKernelGGL(whole_norm_kv_kernel<float>, dim3(rows), dim3(256), 0, (hipStream_t)stream, a);
+  if (is_bf16) hipLaunchKernelGGL(whole_norm_kv_kernel<bf16_t>, dim3(rows, 3), dim3(256), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(whole_norm_kv_kernel<float>, dim3(rows, 3), dim3(256), 0, (hipStream_t)stream, a);
   return BW_LAUNCH_CHECK();
 }
 

@@ -62,7 +62,31 @@ def sepedra_prefill_flops(cfg: dict, tokens: int) -> float:
     return total + 2 * w * cfg["vocab"]
 
 
+def kikarax_prefill_flops(cfg: dict, tokens: int) -> float:
+    """Multiply-adds times two of one prompt: every projection (the output gate's too), the feed-forwards (the router,
+    the chosen experts and the shared one), and the attention's scores and weighted sums over the keys a query sees
+    (its own chunk of positions up to itself)."""
+    w, total = cfg["width"], 0.0
+    for layer in cfg["layers"]:
+        m = layer["mixer"]
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        per_token = w * (H * D + G * (D + V) + H * V) + H * V * w
+        chunk = (m.get("mask") or {}).get("size") or tokens
+        full, rest = divmod(tokens, chunk)
+        pairs = full * chunk * (chunk + 1) / 2 + rest * (rest + 1) / 2
+        mlp = layer.get("mlp")
+        if mlp and mlp["kind"] == "dense":
+            per_token += 3 * w * mlp["ff"]
+        elif mlp:
+            ro = mlp["router"]
+            per_token += w * (ro["experts"] + 1) + ro["top"] * 3 * w * mlp["expert"]["ff"] + 3 * w * (mlp.get("shared") or {"ff": 0})["ff"]
+        total += 2 * (per_token * tokens + H * (D + V) * pairs)
+    return total + 2 * w * cfg["vocab"]
+
+
 def prefill_flops(cfg: dict, tokens: int) -> float:
+    if cfg.get("architecture") == "Kikarax":
+        return kikarax_prefill_flops(cfg, tokens)
     if cfg.get("architecture") == "Kuponex":
         return kuponex_prefill_flops(cfg, tokens)
     if cfg.get("architecture") == "Sepedra":

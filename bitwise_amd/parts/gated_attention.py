@@ -162,12 +162,17 @@ class GatedAttention(Mixer):
     def state_spec(self) -> Optional[StateSpec]:
         return StateSpec(((self.taps - 1) * self.conv_ch,), "float32") if self.taps > 1 else None
 
-    def _run(self, ctx, call, h, target, add: bool) -> None:
+    def _run(self, ctx, call, h, target, add: bool, normed_from=None) -> None:
+        """``normed_from`` = (x, norm) instead of ``h``: the norm rides in the projections' product."""
         rt, ws, rows = self.rt, ctx.ws, ctx.rows
         if self.shared_kv == bool(call.writes_cache):
             raise ValueError("gated_attention: a layer with keys and values of its own writes its cache, one without reads another's")
         proj = ws.buffer("gattn_proj", self.proj.out_features, torch.float32)
-        self.proj.store(ws, h, proj, rows)
+        if normed_from is not None:
+            x, norm = normed_from
+            ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.proj.weight, proj, rows, ops.EPI_F32)
+        else:
+            self.proj.store(ws, h, proj, rows)
         src = proj
         if self.taps >= 1:
             src = ws.buffer("gattn_conv", self.conv_ch, torch.float32)
@@ -213,6 +218,16 @@ class GatedAttention(Mixer):
 
     def forward(self, ctx, call, h, residual) -> None:
         self._run(ctx, call, h, residual, True)
+
+    def forward_with_norm(self, ctx, call, x, norm, residual) -> bool:
+        """Decode steps of few rows: the norm in front of the mixer rides in the stacked projections' product (the bits of
+        norm, then product)."""
+        from .norm import RMSNorm
+        if not (self.rt.bf16 and type(norm) is RMSNorm and self.proj.mfma and self.proj.bias is None
+                and ops.can_fuse_norm(ctx.rows, self.proj.weight, x)):
+            return False
+        self._run(ctx, call, None, residual, True, normed_from=(x, norm))
+        return True
 
     def forward_out(self, ctx, call, h, out) -> None:
         self._run(ctx, call, h, out, False)
