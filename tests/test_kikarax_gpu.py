@@ -62,6 +62,12 @@ CONFIGS = {
     "only_embedding": config(48, 61, 1e-5, 1.0, 5.0, (23, 31, 3), [attn(1, 1, 16, 16, 0.25)]),
     "only_attention": config(48, 61, 1e-5, 1.0, 1.0, None, [attn(4, 2, 16, 8, 0.6, softcap=4.0, chunk=20)]),
     "only_dense": config(48, 61, 1e-5, 2.0, 1.0, None, [attn(1, 1, 16, 16, 0.25, dense(72, 0.4))]),
+    # sizes that are no multiples of 8 anywhere: every product stays on the 32-bit kernels in bfloat16 mode too, heads are
+    # padded in the cache, a pair table of one bucket
+    "odd": config(44, 53, 1e-5, 0.7, 2.0, (1, 3, 2), [
+        attn(3, 1, 20, 12, 0.3, dense(52, 0.8), softcap=5.0, chunk=7, v_mix=True),
+        attn(2, 2, 10, 6, 0.5, moe(5, 2, 20, 3.0, 12), chunk=33, v_mix=True),
+    ]),
     # (experts whose inner size is no multiple of 8 stay on the 32-bit kernels in bfloat16 mode too)
     "only_moe": config(48, 61, 1e-5, 1.0, 1.0, None, [attn(1, 1, 16, 16, 0.25, moe(8, 3, 20, 2.5, 12))]),
     # everything together, sizes all different from layer to layer: values wider and narrower than keys, one key head
