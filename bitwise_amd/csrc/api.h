@@ -35,6 +35,8 @@ int bw_gemm_f32(const float* x, const void* w, int w_is_bf16, float* y, int M, i
                 int accumulate, void* stream);
 int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, int epilogue,
                  void* stream);
+int bw_gemm_clamped_glu_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, float limit,
+                             float alpha, void* stream);
 int bw_gemm_add_scratch(int M, int N, int K, long long* scratch_floats, int* counters);
 int bw_gemm_add_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo, float* scratch,
                      long long scratch_floats, int32_t* counters, int num_counters, void* stream);

@@ -78,6 +78,15 @@ __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp
 // rounded to bfloat16 anyway); one fixed instruction sequence wherever it is used, so every route gives the same bits.
 __device__ __forceinline__ float silu_times(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + fast_exp(-g)) * u; }
 
+// The clamped gated unit g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit), as the 32-bit
+// activation kernel and the products' epilogue both compute it: one sequence of operations, so both give the same bits.
+__device__ __forceinline__ float clamped_swish_times(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit) + 1.0f;
+  const float ag = g * (1.0f / (1.0f + bw_expf(-alpha * g)));
+  return ag * u;
+}
+
 // Lane exchanges from register to register (no trip through LDS).  The halves and quarters of the wave by gfx950's
 // lane swaps: of (v, v) swapped, the first result holds in every lane the value of its partner or its own in the
 // lower half (32: lanes 0-31; 16: the even rows of 16 lanes), the second the one in the upper half; an operation

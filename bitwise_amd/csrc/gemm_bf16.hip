@@ -62,6 +62,7 @@ struct QkvRopeArgs {
   int heads, kv_heads, page_size, table_stride, write_cache;
   int page_shift;              // page_size is a power of two: positions are split by shift and mask, not by division
   int head_dim = 64;           // (the kernels for up to 64 rows take multiples of 64; the tiled ones 64)
+  float glu_limit = 0.0f, glu_alpha = 1.0f;   // EPI_CLAMPED_GLU_BF16 only: the clamp and the sigmoid's slope
 };
 
 // ------------------------------------------------------------------------------ phases of one launch
@@ -127,11 +128,13 @@ __device__ __forceinline__ void st_bf16(bf16_t* p, bf16_t v) {
 }
 
 template <int EPI, bool DEV = false>
-__device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o, float v, float u) {
+__device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o, float v, float u, float limit = 0.0f,
+                                               float alpha = 1.0f) {
   if constexpr (EPI == EPI_F32) st_f32<DEV>((float*)out + o, v);
   else if constexpr (EPI == EPI_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(v));
   else if constexpr (EPI == EPI_ADD_F32) st_f32<DEV>((float*)out + o, ld_f32<DEV>((const float*)out + o) + v);
   else if constexpr (EPI == EPI_SWIGLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(silu_times(v, u)));
+  else if constexpr (EPI == EPI_CLAMPED_GLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(clamped_swish_times(v, u, limit, alpha)));
 }
 
 // (host) The phases asked for while a chain is open wait in a list and leave as one launch (further down).
@@ -254,12 +257,13 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
                             hipStream_t s, const QkvRopeArgs& rp = QkvRopeArgs{}, const MidSplitArgs& sp = MidSplitArgs{},
                             size_t scratch_floats = 0, int num_counters = 0) {
   const int S = (K + GEMM_SEG - 1) / GEMM_SEG;
-  constexpr int NB = (EPI == EPI_SWIGLU_BF16) ? 2 : 1;
+  constexpr int NB = epi_is_glu(EPI) ? 2 : 1;
   if (M <= 64) {
-    if constexpr (EPI == EPI_QKV_ROPE) return -2;       // the rotary epilogue belongs to the wide kernel
+    // (the rotary epilogue belongs to the wide kernel; the clamped unit of few rows is a kernel behind the 32-bit product)
+    if constexpr (EPI == EPI_QKV_ROPE || EPI == EPI_CLAMPED_GLU_BF16) return -2;
     else {
       // one segment and enough columns: the rows of x are shared through LDS
-      constexpr int MID_COLS = (EPI == EPI_SWIGLU_BF16) ? 32 : 64;
+      constexpr int MID_COLS = epi_is_glu(EPI) ? 32 : 64;
       const int wgs = (N + MID_COLS - 1) / MID_COLS;
       // (the descriptors of W cover a tile's rows each, so only the rows of x have to fit 31 bits of offset)
       const bool fits = (size_t)M * ldx * 2 < ((size_t)1 << 31);
@@ -300,7 +304,7 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         }
       }
     }
-    if constexpr (EPI != EPI_SWIGLU_BF16 && EPI != EPI_QKV_ROPE) {
+    if constexpr (!epi_is_glu(EPI) && EPI != EPI_QKV_ROPE) {
       // up to 16 rows: a wave per strip and segment, streaming through its own ring in LDS
       if (M <= 16 && K % 64 == 0 && S <= 40 && (size_t)M * ldx * 2 < ((size_t)1 << 31)) {
         // one segment and few columns: everything asked for at once
@@ -425,12 +429,12 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
     }
     if constexpr (EPI != EPI_ADD_F32) {
       // enough 256-row tiles to go round the compute units (a second round at least half full)
-      constexpr int BIG_COLS = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
+      constexpr int BIG_COLS = epi_is_glu(EPI) ? 128 : 256;
       const int bm = (M + BIG_BM - 1) / BIG_BM, bn = (N + BIG_COLS - 1) / BIG_COLS;
       // (fewer of these tiles than compute units while the 128-row tiles below would fill the chip in one round: a step
       // of those takes half as long, so they win: gate|up of 512 rows 62 us here, half the chip idle)
       bool half_tiles_win = false;
-      if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16) {
+      if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || epi_is_glu(EPI)) {
         const int t256 = ((M + 127) / 128) * bn;
         half_tiles_win = (t256 + 255) / 256 < 2 * ((bm * bn + 255) / 256);
       }
@@ -446,17 +450,17 @@ static int launch_gemm_bf16(const bf16_t* x, const bf16_t* w, void* out, int M, 
         return BW_LAUNCH_CHECK();
       }
     }
-    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || EPI == EPI_SWIGLU_BF16 || EPI == EPI_QKV_ROPE) {
+    if constexpr (EPI == EPI_F32 || EPI == EPI_BF16 || epi_is_glu(EPI) || EPI == EPI_QKV_ROPE) {
       // 128 x 256 tiles where they go round the compute units (the 256 x 256 kernel above took what it takes: one
       // segment of K and enough of its tiles); the q|k|v product of 600 to 1,200 rows among them (four heads of 64 a
       // tile, a head a wave as in the 128 x 128 tiles: 1,024 rows 45.8 us there)
-      constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
+      constexpr int COLS256 = epi_is_glu(EPI) ? 128 : 256;
       const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
       // (in rounds of 256 workgroups; a step of these takes 1.0 us where a 128 x 128 tile's takes 0.58)
       const int rounds256 = (mt * nt + 255) / 256, rounds128 = (mt * ((N + COLS256 / 2 - 1) / (COLS256 / 2)) + 255) / 256;
       if (K % 64 == 0 && 7 * rounds256 <= 4 * rounds128) return launch_tile256<EPI>(x, w, out, M, N, K, ldx, ldo, s, rp);
     }
-    constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
+    constexpr int COLS = epi_is_glu(EPI) ? 64 : 128;
     const int m_tiles = (M + WIDE_BM - 1) / WIDE_BM, n_tiles = (N + COLS - 1) / COLS;
     dim3 grid(m_tiles * n_tiles), block(256);
     {
@@ -537,6 +541,22 @@ extern "C" int bw_gemm_bf16(const void* x, const void* w, void* out, int M, int 
     case EPI_SWIGLU_BF16: return launch_gemm_bf16<EPI_SWIGLU_BF16>(xp, wp, out, M, N, K, ldx, ldo, s);
   }
   return -2;
+}
+
+// The stacked gate|up product of more than 64 rows with the clamped gated unit in its epilogue:
+// out[m, n] = bf16(g' sigmoid(alpha g') (u' + 1)), g' = min(x.W[n], limit), u' = clamp(x.W[N + n], -limit, limit); w is
+// [2N, K].  The bits of gemm_bf16 (32-bit store) + glu.
+extern "C" int bw_gemm_clamped_glu_bf16(const void* x, const void* w, void* out, int M, int N, int K, int ldx, int ldo,
+                                        float limit, float alpha, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M <= 64 || !(limit > 0.0f)) return -2;
+  if (K <= 0 || (K % 8) || (ldx % 8) || ldx < K || ldo < N) return -2;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return -3;
+  QkvRopeArgs rp{};
+  rp.glu_limit = limit;
+  rp.glu_alpha = alpha;
+  return launch_gemm_bf16<EPI_CLAMPED_GLU_BF16>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, ldx, ldo,
+                                                (hipStream_t)stream, rp);
 }
 
 // The stacked q|k|v product with rotation and cache write in its epilogue (heads of 64 elements, K of one

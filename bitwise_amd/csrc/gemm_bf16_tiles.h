@@ -98,11 +98,11 @@ __device__ __forceinline__ void tile_epilogue(const f32x4 (&acc)[NI][4], void* _
             for (int j = 0; j < 4; ++j) dst[(size_t)(16 * j + r) * rp.page_size] = f32_to_bf16(acc[i][j][q]);
           }
         }
-      } else if constexpr (EPI == EPI_SWIGLU_BF16) {
+      } else if constexpr (epi_is_glu(EPI)) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int n = col0 + 16 * j + r;
-          if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j + 2][q]);
+          if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][j][q], acc[i][j + 2][q], rp.glu_limit, rp.glu_alpha);
         }
       } else {
 #pragma unroll
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                              void* __restrict__ out, int M, int N, int K, int ldx,
                                                              int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp) {
   // In SwiGLU mode a block covers 64 output columns: B rows 0-63 are gate rows, 64-127 up rows.
-  constexpr int COLS = (EPI == EPI_SWIGLU_BF16) ? 64 : 128;
+  constexpr int COLS = epi_is_glu(EPI) ? 64 : 128;
   __shared__ __attribute__((aligned(16))) bf16_t lds_a[2][WIDE_BM * WIDE_LDS_ROW];
   __shared__ __attribute__((aligned(16))) bf16_t lds_b[2][WIDE_BN * WIDE_LDS_ROW];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -160,7 +160,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int brow[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    if constexpr (EPI == EPI_SWIGLU_BF16) brow[j] = (j >> 1) * 64 + 32 * wx + 16 * (j & 1);
+    if constexpr (epi_is_glu(EPI)) brow[j] = (j >> 1) * 64 + 32 * wx + 16 * (j & 1);
     else brow[j] = 64 * wx + 16 * j;
   }
 
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       ra[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, voff_a, (32 * j * ldx + k0) * 2, 0);
-      if constexpr (EPI == EPI_SWIGLU_BF16)
+      if constexpr (epi_is_glu(EPI))
         rb[set][j] = __builtin_amdgcn_raw_buffer_load_b128(j < 2 ? rs_b0 : rs_b1, voff_b, (32 * (j & 1) * K + k0) * 2, 0);
       else
         rb[set][j] = __builtin_amdgcn_raw_buffer_load_b128(rs_b0, voff_b, (32 * j * K + k0) * 2, 0);
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = tot[TOT ? i : 0][TOT ? j : 0];
   }
-  tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (EPI == EPI_SWIGLU_BF16 ? 32 : 64) * wx, (n0 >> 6) + wx, r, g,
+  tile_epilogue<EPI, 4>(acc, out, M, N, ldo, m0 + 64 * wy, n0 + (epi_is_glu(EPI) ? 32 : 64) * wx, (n0 >> 6) + wx, r, g,
                         TOT, rp);
 }
 
@@ -359,7 +359,7 @@ template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_big_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
     int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp, size_t seg_stride) {
-  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr bool GLU = epi_is_glu(EPI);
   constexpr int COLS = GLU ? 128 : 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char big_lds[];   // [5 slots][32 KB]
   // gridDim.y > 1: workgroup (tile, y) works on segment y of K alone and leaves its sums at out + y * seg_stride
@@ -608,7 +608,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             unsigned char* row = big_lds + (128 * wy + 16 * i + 4 * g + q) * TROW + (32 * wx + r) * 2;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
-              *reinterpret_cast<bf16_t*>(row + 32 * j) = f32_to_bf16(silu_times(acc[i][j][q], acc[i][j + 2][q]));
+              if constexpr (EPI == EPI_CLAMPED_GLU_BF16)
+                *reinterpret_cast<bf16_t*>(row + 32 * j) =
+                    f32_to_bf16(clamped_swish_times(acc[i][j][q], acc[i][j + 2][q], rp.glu_limit, rp.glu_alpha));
+              else
+                *reinterpret_cast<bf16_t*>(row + 32 * j) = f32_to_bf16(silu_times(acc[i][j][q], acc[i][j + 2][q]));
           }
         __syncthreads();
         const int chunk = threadIdx.x & 15, row0 = threadIdx.x >> 4;
@@ -658,7 +662,7 @@ template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile128_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
     int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp, size_t seg_stride) {
-  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr bool GLU = epi_is_glu(EPI);
   constexpr bool ROPE = EPI == EPI_QKV_ROPE;           // waves of 32 x 64 outputs: a head's 64 columns in one wave
   // gridDim.y > 1: workgroup (tile, y) works on segment y of K alone and leaves its sums at out + y * seg_stride
   // elements (a residual add's segments, joined in order by add_segments_kernel afterwards)
@@ -789,7 +793,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if (m >= M) continue;
       if constexpr (GLU) {
         const int n = n0 + 16 * wx + r;
-        if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][1][q]);
+        if (n < N) epilogue_store<EPI>(out, (size_t)m * ldo + n, acc[i][0][q], acc[i][1][q], rp.glu_limit, rp.glu_alpha);
       } else {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -816,7 +820,7 @@ template <int EPI>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_bf16_tile256_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out, int M, int N, int K, int ldx,
     int ldo, int m_tiles, int n_tiles, QkvRopeArgs rp, size_t seg_stride) {
-  constexpr bool GLU = EPI == EPI_SWIGLU_BF16;
+  constexpr bool GLU = epi_is_glu(EPI);
   constexpr int COLS = GLU ? 128 : 256;
   extern __shared__ __attribute__((aligned(16))) unsigned char t256_lds[];   // [3 stages][x 16 KB | W 32 KB]
   // gridDim.y > 1: workgroup (tile, y) works on segment y of K alone and leaves its sums at out + y * seg_stride
@@ -953,7 +957,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 template <int EPI>
 static int launch_tile256(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K, int ldx, int ldo, hipStream_t s,
                           const QkvRopeArgs& rp = QkvRopeArgs{}, int segments = 1, size_t seg_stride = 0) {
-  constexpr int COLS256 = (EPI == EPI_SWIGLU_BF16) ? 128 : 256;
+  constexpr int COLS256 = epi_is_glu(EPI) ? 128 : 256;
   const int mt = (M + 127) / 128, nt = (N + COLS256 - 1) / COLS256;
   static bool allowed = false;                   // more than 64 KB of dynamic LDS has to be asked for once
   if (!allowed) {

@@ -14,7 +14,10 @@
 #define BW_HD inline
 #endif
 
-enum { EPI_F32 = 0, EPI_BF16 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU_BF16 = 3, EPI_QKV_ROPE = 4 };
+enum { EPI_F32 = 0, EPI_BF16 = 1, EPI_ADD_F32 = 2, EPI_SWIGLU_BF16 = 3, EPI_QKV_ROPE = 4, EPI_CLAMPED_GLU_BF16 = 5 };
+
+// Epilogues that take the stacked weight [gate rows; up rows] and store act(gate) * up.
+BW_HD constexpr bool epi_is_glu(int epi) { return epi == EPI_SWIGLU_BF16 || epi == EPI_CLAMPED_GLU_BF16; }
 
 #define GEMM_SEG 2048                 // a segment of K: sums of different segments are joined left to right
 #define BW_LDS_LIMIT (160 * 1024)     // bytes of LDS a workgroup of gfx950 may ask for

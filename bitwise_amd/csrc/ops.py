@@ -47,6 +47,7 @@ _SIGS = {
                         c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_gemm_f32": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "bw_gemm_clamped_glu_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p],
     "bw_gemm_add_scratch": [c_int, c_int, c_int, c_void_p, c_void_p],
     "bw_gemm_add_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_longlong, c_void_p,
                          c_int, c_void_p],
@@ -461,6 +462,27 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, ep
         return
     _check(_fn("bw_gemm_bf16")(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, N, K, x.stride(0), out.stride(0),
                                epilogue, _stream()), "gemm_bf16")
+
+
+CLAMPED_GLU_MIN_ROWS = 65      # steps of fewer rows run the clamped unit as a kernel behind the 32-bit product
+
+
+def gemm_clamped_glu_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, limit: float, alpha: float) -> None:
+    """out[:rows, n] = bf16(g sigmoid(alpha g) (u + 1)), g = min(x . w[n], limit), u = clamp(x . w[N + n], -limit, limit):
+    the stacked product [2N, K] of a prompt portion (more than 64 rows) with the clamped gated unit in its epilogue; the
+    bits of gemm_bf16 with a 32-bit store followed by ``glu``."""
+    _need(x, torch.bfloat16, "x")
+    _need(w, torch.bfloat16, "weight")
+    _need(out, torch.bfloat16, "out")
+    if w.dim() != 2 or w.shape[0] % 2:
+        raise ValueError("gemm_clamped_glu_bf16: weight must be the stacked [2N, K]")
+    N, K = w.shape[0] // 2, w.shape[1]
+    if x.shape[1] != K or out.shape[1] != N or x.shape[0] < rows or out.shape[0] < rows:
+        raise ValueError(f"gemm_clamped_glu_bf16: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match")
+    if rows < CLAMPED_GLU_MIN_ROWS or K % 8 or not limit > 0:
+        raise ValueError("gemm_clamped_glu_bf16: more than 64 rows, an inner size in multiples of 8 and a positive limit")
+    _check(_fn("bw_gemm_clamped_glu_bf16")(x.data_ptr(), w.data_ptr(), out.data_ptr(), rows, N, K, x.stride(0), out.stride(0),
+                                           float(limit), float(alpha), _stream()), "gemm_clamped_glu_bf16")
 
 
 # ------------------------------------------------------------------------------ decode fusions

@@ -482,18 +482,15 @@ __global__ void glu_kernel(const float* __restrict__ gu, int ldg, OT* __restrict
   const long long row = idx / inter;
   const int c = (int)(idx % inter);
   float g = gu[row * ldg + c], u = gu[row * ldg + inter + c];
-  float ag;
+  float h;
   if (act == ACT_GELU_TANH) {
     const float inner = 0.7978845608028654f * (g + 0.044715f * ((g * g) * g));
-    ag = (0.5f * g) * (1.0f + tanhf(inner));
+    h = ((0.5f * g) * (1.0f + tanhf(inner))) * u;
   } else if (act == ACT_CLAMPED_SWISH) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit) + 1.0f;
-    ag = g * (1.0f / (1.0f + bw_expf(-alpha * g)));
+    h = clamped_swish_times(g, u, limit, alpha);
   } else {
-    ag = g * (1.0f / (1.0f + bw_expf(-g)));
+    h = (g * (1.0f / (1.0f + bw_expf(-g)))) * u;
   }
-  float h = ag * u;
   if (row_gate != nullptr) h *= 1.0f / (1.0f + bw_expf(-row_gate[row * ld_row_gate]));
   store_act(hout + idx, h);
 }

@@ -120,7 +120,9 @@ class ClampedGLU(GeGLU):
 
         g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), y = g sigmoid(alpha g) (u + 1), out = W_down y
 
-    params: width, inter, limit, alpha (1.702), names.  The activation is one 32-bit kernel behind the stacked product."""
+    params: width, inter, limit, alpha (1.702), names.  Prompt portions of more than 64 rows compute the activation in the
+    stacked product's epilogue (bfloat16 mode, weights the matrix cores take); otherwise it is one 32-bit kernel behind the
+    product.  Both are the same sequence of operations on the same 32-bit sums, so a row's bits do not depend on the route."""
 
     act = ops.ACT_CLAMPED_SWISH
 
@@ -132,3 +134,11 @@ class ClampedGLU(GeGLU):
 
     def _act_params(self) -> dict:
         return {"limit": self.limit, "alpha": self.alpha}
+
+    def forward(self, ctx, h, residual) -> None:
+        if self.rt.bf16 and self.gate_up.mfma and self.gate_up.bias is None and ctx.rows >= ops.CLAMPED_GLU_MIN_ROWS:
+            act = ctx.ws.buffer("mlp_h", self.inter, torch.bfloat16)
+            ops.gemm_clamped_glu_bf16(h, self.gate_up.weight, act, ctx.rows, self.limit, self.alpha)
+            self.down.add_into(ctx.ws, act, residual, ctx.rows)
+        else:
+            super().forward(ctx, h, residual)

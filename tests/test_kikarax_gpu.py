@@ -223,6 +223,8 @@ def test_long_decoding(folders, dtype):
     # most of it as one portion (more than 1,024 (row, expert) pairs: the experts' kernel of prompt portions)
     again = run_cut(rp, "y", toks, [300])
     assert pk.logits_error(again, got, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype])
+    # the kernels of prompt portions and those of single tokens leave the same bits
+    assert np.array_equal(again, got)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -412,6 +414,37 @@ def test_clamped_unit_and_row_gate(gpu, act_dtype):
     ops.glu(gu.to(gpu), out, rows, ops.ACT_SILU, row_gate=gu.to(gpu)[:, 2 * inter:2 * inter + 1])
     want = a * torch.sigmoid(a) * b * torch.sigmoid(gu[:, 2 * inter:2 * inter + 1].double())
     assert (out.cpu().double() - want).abs().max() < tol * 4
+
+
+@pytest.mark.parametrize("rows,inter,width", [(65, 64, 64), (130, 136, 72), (200, 1024, 256), (513, 512, 192), (700, 40, 136),
+                                              (1024, 2048, 512), (1500, 96, 2112)])
+def test_clamped_unit_in_the_products_epilogue(gpu, rows, inter, width):
+    """Prompt portions compute the clamped unit in the stacked product's epilogue: the bits of the product's 32-bit sums
+    followed by the activation kernel (what steps of few rows run), over every tiling the product chooses, and the
+    float64 values; inputs large enough for all three clamps to bite."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn(rows, width, generator=g).bfloat16()
+    w = (torch.randn(2 * inter, width, generator=g) * (3.0 / width ** 0.5)).bfloat16()
+    limit, alpha = 1.5, 1.702
+    xd, wd = x.to(gpu), w.to(gpu)
+    fused = torch.zeros(rows, inter, dtype=torch.bfloat16, device=gpu)
+    ops.gemm_clamped_glu_bf16(xd, wd, fused, rows, limit, alpha)
+    sums = torch.zeros(rows, 2 * inter, device=gpu)
+    ops.gemm_bf16(xd, wd, sums, rows, ops.EPI_F32)
+    apart = torch.zeros(rows, inter, dtype=torch.bfloat16, device=gpu)
+    ops.glu(sums, apart, rows, ops.ACT_CLAMPED_SWISH, limit=limit, alpha=alpha)
+    assert torch.equal(fused.view(torch.int16), apart.view(torch.int16))
+    a, b = (x.double() @ w.double().T).split(inter, dim=1)
+    ga = a.clamp(max=limit)
+    want = ga * torch.sigmoid(alpha * ga) * (b.clamp(-limit, limit) + 1.0)
+    assert (a > limit).any() and (b < -limit).any() and (b > limit).any()
+    assert (fused.cpu().double() - want).abs().max() < 3e-2
+    # few rows of the same inputs through the kernel behind the product: the same bits again
+    few = torch.zeros(64, 2 * inter, device=gpu)
+    ops.gemm_bf16(xd[:64].contiguous(), wd, few, 64, ops.EPI_F32)
+    ops.glu(few, apart, 64, ops.ACT_CLAMPED_SWISH, limit=limit, alpha=alpha)
+    assert torch.equal(fused[:64].view(torch.int16), apart[:64].view(torch.int16))
 
 
 def test_router_scale_and_experts_behind_other_columns(gpu):
