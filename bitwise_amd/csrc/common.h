@@ -78,12 +78,17 @@ __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp
 // rounded to bfloat16 anyway); one fixed instruction sequence wherever it is used, so every route gives the same bits.
 __device__ __forceinline__ float silu_times(float g, float u) { return g * __builtin_amdgcn_rcpf(1.0f + fast_exp(-g)) * u; }
 
-// The clamped gated unit g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit), as the 32-bit
+// The clamped gated unit g' sigmoid(alpha g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit), as the
 // activation kernel and the products' epilogue both compute it: one sequence of operations, so both give the same bits.
+// FAST (results that are rounded to bfloat16 anyway): the exponential through the hardware exp2 and the quotient through
+// the hardware reciprocal, as silu_times; otherwise the 32-bit path's exponential and the correctly rounded division.
+template <bool FAST>
 __device__ __forceinline__ float clamped_swish_times(float g, float u, float limit, float alpha) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit) + 1.0f;
-  const float ag = g * (1.0f / (1.0f + bw_expf(-alpha * g)));
+  float ag;
+  if constexpr (FAST) ag = g * __builtin_amdgcn_rcpf(1.0f + fast_exp(-alpha * g));
+  else ag = g * (1.0f / (1.0f + bw_expf(-alpha * g)));
   return ag * u;
 }
 

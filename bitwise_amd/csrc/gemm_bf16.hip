@@ -134,7 +134,7 @@ __device__ __forceinline__ void epilogue_store(void* __restrict__ out, size_t o,
   else if constexpr (EPI == EPI_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(v));
   else if constexpr (EPI == EPI_ADD_F32) st_f32<DEV>((float*)out + o, ld_f32<DEV>((const float*)out + o) + v);
   else if constexpr (EPI == EPI_SWIGLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(silu_times(v, u)));
-  else if constexpr (EPI == EPI_CLAMPED_GLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(clamped_swish_times(v, u, limit, alpha)));
+  else if constexpr (EPI == EPI_CLAMPED_GLU_BF16) st_bf16<DEV>((bf16_t*)out + o, f32_to_bf16(clamped_swish_times<true>(v, u, limit, alpha)));
 }
 
 // (host) The phases asked for while a chain is open wait in a list and leave as one launch (further down).

@@ -610,7 +610,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int j = 0; j < 2; ++j)
               if constexpr (EPI == EPI_CLAMPED_GLU_BF16)
                 *reinterpret_cast<bf16_t*>(row + 32 * j) =
-                    f32_to_bf16(clamped_swish_times(acc[i][j][q], acc[i][j + 2][q], rp.glu_limit, rp.glu_alpha));
+                    f32_to_bf16(clamped_swish_times<true>(acc[i][j][q], acc[i][j + 2][q], rp.glu_limit, rp.glu_alpha));
               else
                 *reinterpret_cast<bf16_t*>(row + 32 * j) = f32_to_bf16(silu_times(acc[i][j][q], acc[i][j + 2][q]));
           }

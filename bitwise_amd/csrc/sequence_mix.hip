@@ -487,7 +487,7 @@ __global__ void glu_kernel(const float* __restrict__ gu, int ldg, OT* __restrict
     const float inner = 0.7978845608028654f * (g + 0.044715f * ((g * g) * g));
     h = ((0.5f * g) * (1.0f + tanhf(inner))) * u;
   } else if (act == ACT_CLAMPED_SWISH) {
-    h = clamped_swish_times(g, u, limit, alpha);
+    h = clamped_swish_times<sizeof(OT) == 2>(g, u, limit, alpha);
   } else {
     h = (g * (1.0f / (1.0f + bw_expf(-g)))) * u;
   }
