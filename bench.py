@@ -146,7 +146,7 @@ def kikarax_shape(width: int, expert_ff: int, pairs: int, experts: int = 32, top
     which a token uses ``top`` beside a shared one), heads of 128 with a quarter as many key heads, chunks of 8,192
     positions, capped scores, values mixed in every layer, a table of 2^16 token pairs and learned positions."""
     heads = width // 128
-    att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+    att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
            "mask": {"size": 8192}, "v_mix": True}
     dense = {"kind": "dense", "ff": 4 * expert_ff, "limit": 7.0}
     moe = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "scale": 2.0}, "shared": {"ff": expert_ff}}
@@ -155,7 +155,7 @@ def kikarax_shape(width: int, expert_ff: int, pairs: int, experts: int = 32, top
         layers.append({"type": "attention", "mixer": dict(att), "mlp": dense})
         layers.append({"type": "attention", "mixer": dict(att), "mlp": moe})
     return {"architecture": "Kikarax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.25,
-            "embedding": {"scale": 16.0, "bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 7}},
+            "embedding": {"scale": 8.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 3}},
             "layers": layers, "max_positions": 16384, "eos_token_id": 2}
 
 

@@ -80,13 +80,13 @@ CONFIGS = {
     "mixed": config(64, 131, 1e-6, 0.3, 7.0, (97, 13, 29), [
         attn(6, 2, 12, 20, 0.5, dense(40, 1.0), softcap=8.0, chunk=37, v_mix=True),
         attn(3, 3, 24, 8, 0.3, moe(6, 1, 40, None, 24)),
-        attn(4, 2, 40, 20, 0.2, None, softcap=30.0, chunk=50, v_mix=True),
+        attn(4, 2, 40, 20, 0.2, None, softcap=35.0, chunk=50, v_mix=True),
         attn(2, 1, 16, 40, 0.4, moe(5, 5, 16, 0.5, None), chunk=16, v_mix=True),
         attn(8, 1, 8, 16, 0.7, dense(24, 3.0), softcap=2.0),
     ]),
     # heads of the sizes real models have, more experts than a wave has lanes, inner sizes beyond one step of the products
-    "wide": config(136, 77, 1e-5, 0.5, 12.0, (509, 127, 7), [
-        attn(4, 4, 128, 128, 0.09, moe(72, 6, 48, 2.0, 64), softcap=30.0, chunk=120, v_mix=True),
+    "wide": config(136, 77, 1e-5, 0.5, 12.0, (251, 59, 3), [
+        attn(4, 4, 128, 128, 0.09, moe(72, 6, 48, 2.0, 64), softcap=25.0, chunk=112, v_mix=True),
         attn(8, 2, 64, 48, 0.12, dense(272, 2.0), softcap=50.0, chunk=64),
         attn(4, 4, 128, 128, 0.05, moe(3, 2, 136, 1.0, 8), chunk=200, v_mix=True),
     ]),
