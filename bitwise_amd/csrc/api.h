@@ -103,19 +103,28 @@ int bw_fingerprint(const float* logits, int vocab, int ld, int rows, const void*
 // Mixers with a fixed-size state per request (sequence_mix.hip).  seq_rows: [requests, 2] = (first row, rows) of every
 // request of the step; slots: its state slot.  A request without rows, with a negative slot or a negative first
 // position is padding: its state stays as it is.
+// mix: [nmix, dim]; out: [rows, >= nmix*dim], block m of a row is the row shifted with mix[m]
 int bw_norm_shift(const float* x, int ldx, const float* w, const float* mix, float* state, long long state_ld,
                   const int32_t* positions, const int32_t* row_seq, const int32_t* seq_rows, const int32_t* slots,
-                  void* out, int out_is_bf16, int ldo, int rows, int dim, float eps, void* stream);
+                  void* out, int out_is_bf16, int ldo, int rows, int dim, float eps, int nmix, void* stream);
 // mode 0: a decay per key channel (gate: logits [rows, ldg] at gate_off, bias [heads*dim], param = 1/tau);
 // mode 1: scalar input and forget gates per head (columns gate_off and gate2_off of proj, biases bias and bias2, param = cap)
 // with normaliser and running maximum.  state: [slots, state_ld] of S [heads][dim][vdim] (mode 1: then n [heads][dim], m [heads]).
+// mode 2: a decay per key channel exp(-exp(logit + bias)), the read-out taken before the update with the token's own
+// k v^T weighted by bias2 [heads*dim]; mode 3: one constant decay a head, bias [heads] (gate is not read).
+// q is multiplied by qscale, k by kscale.
 int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_off, int k_off, int v_off, const float* gate, int ldg,
                          int gate_off, int gate2_off, const float* bias, const float* bias2, float param, float qscale,
-                         float* state, long long state_ld, float* out, int ldo, const int32_t* seq_rows,
+                         float kscale, float* state, long long state_ld, float* out, int ldo, const int32_t* seq_rows,
                          const int32_t* slots, const int32_t* positions, int nseq, int heads, int dim, int vdim,
                          const int32_t* chunks, int nchunks, const int32_t* spans, int nspans, float* scan_local,
                          float* scan_start, long long scan_floats, void* stream);
 // gate 0: sigmoid, 1: SiLU.  weight: [heads, wstride] (wstride 0: one weight vector for all heads).
+// Up to two sections of [heads][dim] 32-bit elements a row (at columns off0, off1) turned in place: of a head's first rot
+// elements, element i is paired with element i + rot/2; tables [positions, rot/2].
+int bw_rotate_halves_rows(float* x, int ldx, int rows, int heads, int dim, int rot, int sections, int off0, int off1,
+                          const float* cos_table, const float* sin_table, const int32_t* positions, void* stream);
+int bw_tanh_rows(float* x, int ld, int rows, int cols, void* stream);      // x <- tanh(x)
 int bw_head_norm_gate(const float* o, int ldi, const float* weight, int wstride, const float* g, int ldg, int gate, void* out,
                       int out_is_bf16, int ldo, const int32_t* positions, int rows, int heads, int vdim, float eps,
                       void* stream);
@@ -151,7 +160,9 @@ int bw_pair_rope_unit(const float* src, int lds, const int32_t* positions, const
                       const int32_t* block_table, int table_stride, const float* cos_table, const float* sin_table,
                       void* q_out, void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads,
                       int dim, int vdim, int hd, int rot, int page_size, int unit_norm, float eps, int has_kv,
-                      int write_cache, void* stream);
+                      int write_cache, int halves, int v_from_k, void* stream);
+// (halves 1: pair i of the rotation is elements (i, i + rot/2) instead of (2i, 2i+1); v_from_k 1: src holds no values, a
+// value head is its key head as projected, before rotation)
 // Queries and keys normed over their whole projection (all heads at once): x / sqrt(mean(x^2) + eps) * w; values as they
 // are or mixed with another layer's values of the same row, v <- (1 - lambda) v + lambda v_first (lambda: one number on
 // the device); the cache write and the queries' copy as bw_pair_rope_unit.  src: [q | k | v] at columns 0, heads*dim,
@@ -161,25 +172,33 @@ int bw_whole_norm_kv(const float* src, int lds, const int32_t* positions, const 
                      const float* v_first, int ldf, const float* lambda, float* v_keep, int ldk, void* q_out,
                      void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads, int dim, int vdim,
                      int hd, int page_size, int write_cache, void* stream);
+// per_head 1: g holds one logit a head ([rows, heads]) instead of one an element
 int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
-                int ldo, int rows, int heads, int vdim, void* stream);
+                int ldo, int rows, int heads, int vdim, int per_head, void* stream);
 // (y and gates are overwritten: y by its activation, the gates' logits by the recurrence's factor and addend)
 int bw_rglru_scan(float* y, int ldy, const float* y_bias, const float* u, int ldu, float* gates, int ldg, const float* ra_bias,
                   const float* ri_bias, const float* decay, float* state, long long state_ld, void* out,
                   int out_is_bf16, int ldo, const int32_t* seq_rows, const int32_t* slots, const int32_t* positions,
                   int nseq, int rows, int channels, int bs, void* stream);
 // place, wts, top (optional): row r of the normed operand is sum_j wts[r][j] * y[place[r][j]] instead of y[r]
+// scale: the normed row is multiplied by it on its way into x (1: added as it is)
 int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
-                int rows, int dim, float eps, const int32_t* place, const float* wts, int top, void* stream);
+                int rows, int dim, float eps, const int32_t* place, const float* wts, int top, float scale, void* stream);
+// out[r] = (1/n) sum_b norm(y[b][r]) * w[b], n <= 4 (host arrays of device pointers)
+int bw_norm_mean(const float* const* y, const int* ldy, const float* const* w, int n, float* out, int ldo, int rows, int dim,
+                 float eps, void* stream);
 int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream);
 int bw_scale_rows(float* x, int ld, int rows, int cols, float factor, void* stream);      // x *= factor
 // A feed-forward of routed experts (moe.hip).
 // (weight_scale: the chosen scores are multiplied by it on their way into wts)
+// score_kind 0: softmax over the experts, 1: sigmoid of each logit; correction (optional, [experts]): added to the scores
+// for the choice only; group_best: a group's score is the sum of that many of its best choice scores (1 to 4)
 int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, float weight_scale,
-                 int32_t* ids, float* wts, void* stream);
+                 int score_kind, const float* correction, int group_best, int32_t* ids, float* wts, void* stream);
 // route, then plan; one launch for steps of up to 16 rows
 int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, float weight_scale,
-                      int32_t* ids, float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream);
+                      int score_kind, const float* correction, int group_best, int32_t* ids, float* wts, int32_t* sorted,
+                      int32_t* place, int32_t* tiles, int32_t* meta, void* stream);
 int bw_moe_max_tiles(int slots, int experts);
 int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* sorted, int32_t* place, int32_t* tiles,
                 int32_t* meta, void* stream);

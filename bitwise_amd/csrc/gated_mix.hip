@@ -139,6 +139,8 @@ struct PairRopeArgs {
   void* v_cache;
   int lds, rows, heads, kv_heads, dim, vdim, hd, rot, page_size, table_stride, unit_norm, has_kv, write_cache;
   float eps;
+  int halves;                  // 0: pair i of the rotation is elements (2i, 2i+1); 1: elements (i, i + rot/2)
+  int v_from_k;                // 1: src holds no values; a value head is the key head as projected (vdim == dim)
 };
 
 // A wave a (row, head): q heads, then k heads, then v heads.  Lane l owns the pairs l, l + 64, ...
@@ -157,7 +159,8 @@ __global__ __launch_bounds__(256) void pair_rope_unit_kernel(PairRopeArgs a) {
   if (!is_q && !is_k) {
     // values: as they are, padded with zeros to the cache's head size
     const int h = hh - a.heads - a.kv_heads;
-    const float* v = a.src + (size_t)row * a.lds + (size_t)(a.heads + a.kv_heads) * a.dim + (size_t)h * a.vdim;
+    const float* v = a.v_from_k ? a.src + (size_t)row * a.lds + (size_t)(a.heads + h) * a.dim
+                                : a.src + (size_t)row * a.lds + (size_t)(a.heads + a.kv_heads) * a.dim + (size_t)h * a.vdim;
     T* vc = reinterpret_cast<T*>(a.v_cache);
     for (int d = lane; d < a.hd; d += 64) {
       const float val = d < a.vdim ? v[d] : 0.0f;
@@ -178,7 +181,9 @@ __global__ __launch_bounds__(256) void pair_rope_unit_kernel(PairRopeArgs a) {
     const int p = lane + 64 * j;
     e0[j] = e1[j] = 0.0f;
     if (p < pairs) {
-      const float x1 = v[2 * p], x2 = 2 * p + 1 < a.dim ? v[2 * p + 1] : 0.0f;
+      // (pairs behind the rotated ones are neighbours in either layout)
+      const int i1 = a.halves && p < half ? p : 2 * p, i2 = a.halves && p < half ? p + half : 2 * p + 1;
+      const float x1 = v[i1], x2 = i2 < a.dim ? v[i2] : 0.0f;
       if (p < half) {
         const float c = ct[p], s = st[p];
         e0[j] = x1 * c - x2 * s;
@@ -202,8 +207,9 @@ __global__ __launch_bounds__(256) void pair_rope_unit_kernel(PairRopeArgs a) {
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int p = lane + 64 * j;
-    if (2 * p < a.hd) gm_store(dst + 2 * p, 2 * p < a.dim ? e0[j] * inv : 0.0f);
-    if (2 * p + 1 < a.hd) gm_store(dst + 2 * p + 1, 2 * p + 1 < a.dim ? e1[j] * inv : 0.0f);
+    const int i1 = a.halves && p < half ? p : 2 * p, i2 = a.halves && p < half ? p + half : 2 * p + 1;
+    if (i1 < a.hd) gm_store(dst + i1, i1 < a.dim ? e0[j] * inv : 0.0f);
+    if (i2 < a.hd) gm_store(dst + i2, i2 < a.dim ? e1[j] * inv : 0.0f);
   }
 }
 
@@ -211,11 +217,12 @@ extern "C" int bw_pair_rope_unit(const float* src, int lds, const int32_t* posit
                                  const int32_t* block_table, int table_stride, const float* cos_table, const float* sin_table,
                                  void* q_out, void* k_cache, void* v_cache, int is_bf16, int rows, int heads, int kv_heads,
                                  int dim, int vdim, int hd, int rot, int page_size, int unit_norm, float eps, int has_kv,
-                                 int write_cache, void* stream) {
+                                 int write_cache, int halves, int v_from_k, void* stream) {
   if (rows <= 0) return 0;
   if (dim > 256 || hd > 256 || dim > hd || vdim > hd || rot % 2 || rot > dim || page_size <= 0) return -2;
+  if (v_from_k && vdim != dim) return -2;
   PairRopeArgs a{src, positions, row_seq, block_table, cos_table, sin_table, q_out, k_cache, v_cache, lds, rows, heads, kv_heads,
-                 dim, vdim, hd, rot, page_size, table_stride, unit_norm, has_kv, write_cache, eps};
+                 dim, vdim, hd, rot, page_size, table_stride, unit_norm, has_kv, write_cache, eps, halves, v_from_k};
   const long long items = (long long)rows * (heads + (has_kv ? 2 * kv_heads : 0));
   const dim3 grid((unsigned)((items + 3) / 4));
   if (is_bf16) hipLaunchKernelGGL(pair_rope_unit_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, a);
@@ -326,29 +333,29 @@ extern "C" int bw_whole_norm_kv(const float* src, int lds, const int32_t* positi
 
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gate_mul_kernel(const TI* __restrict__ av, int lda, int hd, const float* __restrict__ g, int ldg,
-                                                       TO* __restrict__ out, int ldo, int rows, int heads, int vdim) {
+                                                       TO* __restrict__ out, int ldo, int rows, int heads, int vdim, int per_head) {
   const int row = blockIdx.y;
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= heads * vdim) return;
   const int h = e / vdim, d = e % vdim;
   const float x = gm_load(av + (size_t)row * lda + (size_t)h * hd + d);
-  gm_store(out + (size_t)row * ldo + e, x * gm_sigmoid(g[(size_t)row * ldg + e]));
+  gm_store(out + (size_t)row * ldo + e, x * gm_sigmoid(g[(size_t)row * ldg + (per_head ? h : e)]));
 }
 
 extern "C" int bw_gate_mul(const void* av, int a_is_bf16, int lda, int hd, const float* g, int ldg, void* out, int out_is_bf16,
-                           int ldo, int rows, int heads, int vdim, void* stream) {
+                           int ldo, int rows, int heads, int vdim, int per_head, void* stream) {
   if (rows <= 0) return 0;
   if (rows > 65535 * 16) return -2;
   const dim3 grid((heads * vdim + 255) / 256, rows);
   hipStream_t s = (hipStream_t)stream;
   if (a_is_bf16 && out_is_bf16)
-    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)av, lda, hd, g, ldg, (bf16_t*)out, ldo, rows, heads, vdim);
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)av, lda, hd, g, ldg, (bf16_t*)out, ldo, rows, heads, vdim, per_head);
   else if (a_is_bf16)
-    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, float>), grid, dim3(256), 0, s, (const bf16_t*)av, lda, hd, g, ldg, (float*)out, ldo, rows, heads, vdim);
+    hipLaunchKernelGGL((gate_mul_kernel<bf16_t, float>), grid, dim3(256), 0, s, (const bf16_t*)av, lda, hd, g, ldg, (float*)out, ldo, rows, heads, vdim, per_head);
   else if (out_is_bf16)
-    hipLaunchKernelGGL((gate_mul_kernel<float, bf16_t>), grid, dim3(256), 0, s, (const float*)av, lda, hd, g, ldg, (bf16_t*)out, ldo, rows, heads, vdim);
+    hipLaunchKernelGGL((gate_mul_kernel<float, bf16_t>), grid, dim3(256), 0, s, (const float*)av, lda, hd, g, ldg, (bf16_t*)out, ldo, rows, heads, vdim, per_head);
   else
-    hipLaunchKernelGGL((gate_mul_kernel<float, float>), grid, dim3(256), 0, s, (const float*)av, lda, hd, g, ldg, (float*)out, ldo, rows, heads, vdim);
+    hipLaunchKernelGGL((gate_mul_kernel<float, float>), grid, dim3(256), 0, s, (const float*)av, lda, hd, g, ldg, (float*)out, ldo, rows, heads, vdim, per_head);
   return BW_LAUNCH_CHECK();
 }
 
@@ -460,7 +467,8 @@ extern "C" int bw_rglru_scan(float* y, int ldy, const float* y_bias, const float
 template <typename WT>
 __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__ y, int ldy, const WT* __restrict__ w, float* __restrict__ x,
                                                        int ldx, bf16_t* __restrict__ rounded, int ldr, int dim, float eps,
-                                                       const int32_t* __restrict__ place, const float* __restrict__ wts, int top) {
+                                                       const int32_t* __restrict__ place, const float* __restrict__ wts, int top,
+                                                       float scale) {
   __shared__ float part[4];
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* yr = y + (size_t)row * ldy;
@@ -498,14 +506,16 @@ __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__
     for (int j = 0; j < MAXV; ++j) {
       const int e = tid + 256 * j;
       if (e < dim) {
-        const float nx = xr[e] + (v[j] * inv) * gm_load(w + e);
+        const float normed = (v[j] * inv) * gm_load(w + e);
+        const float nx = scale == 1.0f ? xr[e] + normed : fmaf(scale, normed, xr[e]);
         xr[e] = nx;
         if (rounded != nullptr) rounded[(size_t)row * ldr + e] = f32_to_bf16(nx);
       }
     }
   } else {
     for (int e = tid; e < dim; e += 256) {
-      const float nx = xr[e] + (value(e) * inv) * gm_load(w + e);
+      const float normed = (value(e) * inv) * gm_load(w + e);
+      const float nx = scale == 1.0f ? xr[e] + normed : fmaf(scale, normed, xr[e]);
       xr[e] = nx;
       if (rounded != nullptr) rounded[(size_t)row * ldr + e] = f32_to_bf16(nx);
     }
@@ -513,13 +523,69 @@ __global__ __launch_bounds__(256) void norm_add_kernel(const float* __restrict__
 }
 
 extern "C" int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x, int ldx, void* rounded, int ldr,
-                           int rows, int dim, float eps, const int32_t* place, const float* wts, int top, void* stream) {
+                           int rows, int dim, float eps, const int32_t* place, const float* wts, int top, float scale, void* stream) {
   if (rows <= 0) return 0;
   const dim3 grid(rows);
   if (w_is_bf16)
-    hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps, place, wts, top);
+    hipLaunchKernelGGL(norm_add_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const bf16_t*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps, place, wts, top, scale);
   else
-    hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps, place, wts, top);
+    hipLaunchKernelGGL(norm_add_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, y, ldy, (const float*)w, x, ldx, (bf16_t*)rounded, ldr, dim, eps, place, wts, top, scale);
+  return BW_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------ the mean of normed branches
+
+// out[r] = (1/n) sum_b (y_b[r] / sqrt(mean(y_b[r]^2) + eps)) * w_b, b ascending: what mixers that run side by side leave,
+// each normed over the model width with a weight of its own.  A workgroup a row, the sums of squares as in norm_add_kernel.
+struct NormMeanArgs {
+  const float* y[4];
+  const float* w[4];
+  int ldy[4];
+  int n;
+  float* out;
+  int ldo, dim;
+  float eps;
+};
+
+__global__ __launch_bounds__(256) void norm_mean_kernel(NormMeanArgs a) {
+  __shared__ float part[4][4];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  for (int b = 0; b < a.n; ++b) {
+    const float* yr = a.y[b] + (size_t)row * a.ldy[b];
+    float acc = 0.0f;
+    for (int e = tid; e < a.dim; e += 256) acc = fmaf(yr[e], yr[e], acc);
+    acc = wave_sum(acc);
+    if ((tid & 63) == 0) part[b][tid >> 6] = acc;
+  }
+  __syncthreads();
+  float inv[4];
+  for (int b = 0; b < a.n; ++b)
+    inv[b] = 1.0f / sqrtf((((part[b][0] + part[b][1]) + part[b][2]) + part[b][3]) / (float)a.dim + a.eps);
+  const float share = 1.0f / (float)a.n;
+  for (int e = tid; e < a.dim; e += 256) {
+    float sum = 0.0f;
+    for (int b = 0; b < a.n; ++b) sum += (a.y[b][(size_t)row * a.ldy[b] + e] * inv[b]) * a.w[b][e];
+    a.out[(size_t)row * a.ldo + e] = sum * share;
+  }
+}
+
+extern "C" int bw_norm_mean(const float* const* y, const int* ldy, const float* const* w, int n, float* out, int ldo, int rows,
+                            int dim, float eps, void* stream) {
+  if (rows <= 0) return 0;
+  if (n < 1 || n > 4 || dim <= 0 || ldo < dim) return -2;
+  NormMeanArgs a{};
+  for (int b = 0; b < n; ++b) {
+    if (y[b] == nullptr || w[b] == nullptr || ldy[b] < dim) return -2;
+    a.y[b] = y[b];
+    a.w[b] = w[b];
+    a.ldy[b] = ldy[b];
+  }
+  a.n = n;
+  a.out = out;
+  a.ldo = ldo;
+  a.dim = dim;
+  a.eps = eps;
+  hipLaunchKernelGGL(norm_mean_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, a);
   return BW_LAUNCH_CHECK();
 }
 

@@ -1,9 +1,10 @@
 // A feed-forward of routed experts.
 //
-//   route:    per row, scores = softmax of the router's logits over all experts; experts lie in equal groups of
-//             neighbours, a group's score is its best expert's, only experts of the `keep` best groups can be chosen;
-//             the `top` best of those are the row's experts, weighted by their scores as they are.  Ties go to the
-//             lower index.  All 32-bit.
+//   route:    per row, scores = softmax of the router's logits over all experts, or the sigmoid of each; the choice is
+//             made on the scores, or on the scores plus a learned correction per expert; experts lie in equal groups of
+//             neighbours, a group's score is its best choice score (or the sum of its few best), only experts of the
+//             `keep` best groups can be chosen; the `top` best of those are the row's experts, weighted by their scores
+//             (without the correction) as they are.  Ties go to the lower index.  All 32-bit.
 //   plan:     the step's (row, choice) pairs ("slots") sorted by expert into runs, and the runs cut into tiles of
 //             16 or 128 slots (steps of few or of many slots): every tile belongs to one expert.  Built on the device; the products' grids are sized for
 //             the worst case and tiles past the last return at once.
@@ -39,79 +40,108 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// A wave a row.  LDS of the wave: scores [E], group scores [count], allowed [count].
+// How a row's experts are scored and chosen.  kind 0: scores are the softmax of the logits over all experts; kind 1: the
+// sigmoid of each logit.  correction (optional, [E]): the choice is made on score + correction, the weights stay the scores.
+// group_best: a group's score is the sum of its group_best largest choice scores (1: its best expert's).
+struct RouteRule {
+  int kind;
+  const float* correction;
+  int group_best;
+};
+
+// A wave a row.  LDS of the wave: scores [E], choice scores [E], group scores [count], allowed [count].
 __device__ __forceinline__ void route_row(const float* __restrict__ logits, int ld, int row, int E, int top, int count, int keep,
-                                          float weight_scale, int32_t* __restrict__ ids, float* __restrict__ wts, float* s, int lane) {
-  float* gs = s + E;
+                                          float weight_scale, RouteRule rule, int32_t* __restrict__ ids, float* __restrict__ wts,
+                                          float* s, int lane) {
+  float* c = s + E;
+  float* gs = c + E;
   float* allowed = gs + count;
   const float* z = logits + (size_t)row * ld;
-  float mx = -INFINITY;
-  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-  mx = wave_max(mx);
-  float sum = 0.0f;
-  for (int e = lane; e < E; e += 64) {
-    const float ex = bw_expf(z[e] - mx);
-    s[e] = ex;
-    sum += ex;
+  if (rule.kind == 1) {
+    for (int e = lane; e < E; e += 64) s[e] = 1.0f / (1.0f + bw_expf(-z[e]));
+  } else {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) {
+      const float ex = bw_expf(z[e] - mx);
+      s[e] = ex;
+      sum += ex;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) s[e] = s[e] / sum;
   }
-  sum = wave_sum(sum);
-  for (int e = lane; e < E; e += 64) s[e] = s[e] / sum;
+  for (int e = lane; e < E; e += 64) c[e] = rule.correction != nullptr ? s[e] + rule.correction[e] : s[e];
   __builtin_amdgcn_wave_barrier();
   const int gsz = E / count;
   for (int g = lane; g < count; g += 64) {
-    float best = -1.0f;
-    for (int j = 0; j < gsz; ++j) best = fmaxf(best, s[g * gsz + j]);
-    gs[g] = best;
+    // the group's largest choice scores, one after the other (lower index first among equals), added in that order
+    float total = 0.0f;
+    int taken[4] = {-1, -1, -1, -1};
+    const int nbest = min(min(rule.group_best, gsz), 4);
+    for (int b = 0; b < nbest; ++b) {
+      float best = -INFINITY;
+      int at = -1;
+      for (int j = 0; j < gsz; ++j) {
+        if (j == taken[0] || j == taken[1] || j == taken[2] || j == taken[3]) continue;
+        if (at < 0 || c[g * gsz + j] > best) { best = c[g * gsz + j]; at = j; }
+      }
+      taken[b] = at;
+      total = b == 0 ? best : total + best;
+    }
+    gs[g] = total;
     allowed[g] = keep >= count ? 1.0f : 0.0f;
   }
   __builtin_amdgcn_wave_barrier();
   if (keep < count) {
     for (int it = 0; it < keep; ++it) {
-      float v = -2.0f;
+      float v = -INFINITY;
       int i = 0x7fffffff;
       for (int g = lane; g < count; g += 64)
-        if (gs[g] > v) { v = gs[g]; i = g; }
+        if (allowed[g] == 0.0f && (i == 0x7fffffff || gs[g] > v)) { v = gs[g]; i = g; }
       wave_argmax(v, i);
-      if (lane == 0) { gs[i] = -3.0f; allowed[i] = 1.0f; }
+      if (lane == 0) allowed[i] = 1.0f;
       __builtin_amdgcn_wave_barrier();
     }
   }
+  // (a chosen expert's choice score becomes NaN: no comparison takes it again)
   for (int it = 0; it < top; ++it) {
-    float v = -2.0f;
+    float v = -INFINITY;
     int i = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float sc = allowed[e / gsz] > 0.0f ? s[e] : -2.0f;
-      if (sc > v) { v = sc; i = e; }
+      const bool open = allowed[e / gsz] > 0.0f && c[e] == c[e];
+      if (open && (i == 0x7fffffff || c[e] > v)) { v = c[e]; i = e; }
     }
     wave_argmax(v, i);
     if (lane == 0) {
       ids[(size_t)row * top + it] = i;
-      wts[(size_t)row * top + it] = v * weight_scale;
-      s[i] = -3.0f;
+      wts[(size_t)row * top + it] = s[i] * weight_scale;
+      c[i] = __builtin_nanf("");
     }
     __builtin_amdgcn_wave_barrier();
   }
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
-                                                        int keep, float weight_scale, int32_t* __restrict__ ids,
+                                                        int keep, float weight_scale, RouteRule rule, int32_t* __restrict__ ids,
                                                         float* __restrict__ wts) {
   extern __shared__ float route_lds[];
   const int wave = wave_index(), lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + wave;
   if (row >= rows) return;
-  route_row(logits, ld, row, E, top, count, keep, weight_scale, ids, wts, route_lds + (size_t)wave * (E + 2 * count), lane);
+  route_row(logits, ld, row, E, top, count, keep, weight_scale, rule, ids, wts, route_lds + (size_t)wave * (2 * E + 2 * count), lane);
 }
 
 extern "C" int bw_moe_route(const float* logits, int ld, int rows, int experts, int top, int groups, int keep, float weight_scale,
-                            int32_t* ids, float* wts, void* stream) {
+                            int score_kind, const float* correction, int group_best, int32_t* ids, float* wts, void* stream) {
   if (rows <= 0) return 0;
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || groups < 1 || experts % groups || keep < 1 || keep > groups ||
-      top > keep * (experts / groups))
+      top > keep * (experts / groups) || score_kind < 0 || score_kind > 1 || group_best < 1 || group_best > 4)
     return -2;
-  const size_t bytes = (size_t)4 * (experts + 2 * groups) * sizeof(float);
+  const size_t bytes = (size_t)4 * (2 * experts + 2 * groups) * sizeof(float);
   hipLaunchKernelGGL(moe_route_kernel, dim3((rows + 3) / 4), dim3(256), bytes, (hipStream_t)stream, logits, ld, rows, experts, top,
-                     groups, keep, weight_scale, ids, wts);
+                     groups, keep, weight_scale, RouteRule{score_kind, correction, group_best}, ids, wts);
   return BW_LAUNCH_CHECK();
 }
 
@@ -194,14 +224,14 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
 
 // Steps of up to 16 rows: route (a wave a row) and plan in one launch of one workgroup.
 __global__ __launch_bounds__(1024) void moe_route_plan_kernel(const float* __restrict__ logits, int ld, int rows, int E, int top, int count,
-                                                              int keep, float weight_scale, int32_t* __restrict__ ids, float* __restrict__ wts, int segs,
+                                                              int keep, float weight_scale, RouteRule rule, int32_t* __restrict__ ids, float* __restrict__ wts, int segs,
                                                               int tm, int32_t* __restrict__ sorted, int32_t* __restrict__ place,
                                                               int32_t* __restrict__ tiles, int32_t* __restrict__ meta) {
   extern __shared__ float both_lds[];   // the waves' routing tables, then the plan's slots
   const int wave = wave_index(), lane = threadIdx.x & 63;
-  if (wave < rows) route_row(logits, ld, wave, E, top, count, keep, weight_scale, ids, wts, both_lds + (size_t)wave * (E + 2 * count), lane);
+  if (wave < rows) route_row(logits, ld, wave, E, top, count, keep, weight_scale, rule, ids, wts, both_lds + (size_t)wave * (2 * E + 2 * count), lane);
   __syncthreads();                      // (the rows' choices, written to memory by their waves, are visible to the workgroup)
-  plan_body(ids, rows * top, E, segs, tm, 1, reinterpret_cast<int*>(both_lds + (size_t)rows * (E + 2 * count)), sorted, place, tiles, meta);
+  plan_body(ids, rows * top, E, segs, tm, 1, reinterpret_cast<int*>(both_lds + (size_t)rows * (2 * E + 2 * count)), sorted, place, tiles, meta);
 }
 
 // Slots a tile: few slots a step (decoded tokens) get tiles of 16, whose kernel keeps many steps of weights in flight;
@@ -225,18 +255,19 @@ extern "C" int bw_moe_plan(const int32_t* ids, int slots, int experts, int32_t* 
 }
 
 extern "C" int bw_moe_route_plan(const float* logits, int ld, int rows, int experts, int top, int groups, int keep,
-                                 float weight_scale, int32_t* ids, float* wts, int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream) {
+                                 float weight_scale, int score_kind, const float* correction, int group_best, int32_t* ids, float* wts,
+                                 int32_t* sorted, int32_t* place, int32_t* tiles, int32_t* meta, void* stream) {
   if (rows <= 0) return 0;
-  const size_t bytes = ((size_t)rows * (experts + 2 * groups) + (size_t)rows * top) * sizeof(float);
+  const size_t bytes = ((size_t)rows * (2 * experts + 2 * groups) + (size_t)rows * top) * sizeof(float);
   if (rows > 16 || bytes > 48 * 1024) {
-    const int rc = bw_moe_route(logits, ld, rows, experts, top, groups, keep, weight_scale, ids, wts, stream);
+    const int rc = bw_moe_route(logits, ld, rows, experts, top, groups, keep, weight_scale, score_kind, correction, group_best, ids, wts, stream);
     return rc != 0 ? rc : bw_moe_plan(ids, rows * top, experts, sorted, place, tiles, meta, stream);
   }
   if (experts < 1 || experts > MOE_MAX_EXPERTS || top < 1 || groups < 1 || experts % groups || keep < 1 || keep > groups ||
-      top > keep * (experts / groups))
+      top > keep * (experts / groups) || score_kind < 0 || score_kind > 1 || group_best < 1 || group_best > 4)
     return -2;
   hipLaunchKernelGGL(moe_route_plan_kernel, dim3(1), dim3(1024), bytes, (hipStream_t)stream, logits, ld, rows, experts, top, groups, keep,
-                     weight_scale, ids, wts, 1024 / experts, bw_moe_tile_rows(rows * top), sorted, place, tiles, meta);
+                     weight_scale, RouteRule{score_kind, correction, group_best}, ids, wts, 1024 / experts, bw_moe_tile_rows(rows * top), sorted, place, tiles, meta);
   return BW_LAUNCH_CHECK();
 }
 

@@ -8,7 +8,7 @@ from __future__ import annotations
 import ctypes
 import functools
 from ctypes import c_double, c_float, c_int, c_longlong, c_void_p
-from typing import Optional, Tuple
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -78,9 +78,12 @@ _SIGS = {
     "bw_sample": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_fingerprint": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "bw_norm_shift": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
-                      c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
+                      c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "bw_rotate_halves_rows": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
+    "bw_tanh_rows": [c_void_p, c_int, c_int, c_int, c_void_p],
+    "bw_norm_mean": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "bw_linear_recurrence": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
-                             c_float, c_float, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                             c_float, c_float, c_float, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                              c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p],
     "bw_head_norm_gate": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
                           c_int, c_int, c_float, c_void_p],
@@ -102,17 +105,17 @@ _SIGS = {
                        c_void_p, c_int, c_int, c_void_p, c_int, c_void_p],
     "bw_pair_rope_unit": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
-                          c_int, c_void_p],
-    "bw_gate_mul": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+                          c_int, c_int, c_int, c_void_p],
+    "bw_gate_mul": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "bw_rglru_scan": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
                       c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "bw_norm_add": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p, c_void_p,
-                    c_int, c_void_p],
+                    c_int, c_float, c_void_p],
     "bw_softcap": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
     "bw_scale_rows": [c_void_p, c_int, c_int, c_int, c_float, c_void_p],
-    "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p],
-    "bw_moe_route_plan": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                          c_void_p, c_void_p],
+    "bw_moe_route": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    "bw_moe_route_plan": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_moe_max_tiles": [c_int, c_int],
     "bw_moe_plan": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_moe_experts": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -408,11 +411,11 @@ def rope_kvwrite(qkv: torch.Tensor, q_out: Optional[torch.Tensor], positions: to
 # ------------------------------------------------------------------------------ matrix products
 
 def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, accumulate: bool = False) -> None:
-    """out[:rows] (+)= x[:rows] @ w.T with one k-ascending fused multiply-add chain per output.  ``x`` may be a
-    column slice of a wider matrix (rows apart by its stride)."""
+    """out[:rows] (+)= x[:rows] @ w.T with one k-ascending fused multiply-add chain per output.  ``x`` and ``out`` may
+    be column slices of wider matrices (rows apart by their strides)."""
     if not x.is_cuda or x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
         raise ValueError("gemm_f32: x must be a float32 GPU matrix with contiguous rows")
-    _need(out, torch.float32, "out")
+    _need_strided(out, torch.float32, "out")
     if not w.is_cuda or not w.is_contiguous() or w.dim() != 2:
         raise ValueError("gemm_f32: weight must be a contiguous [N, K] GPU tensor")
     N, K = w.shape
@@ -437,8 +440,9 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, ep
     """out[:rows] = epilogue(x[:rows] @ w.T) on the matrix cores; see gemm_bf16.hip for the
     arithmetic.  EPI_SWIGLU_BF16 takes the stacked weight [2N, K] (gate rows, then up rows).
     ``scratch`` (EPI_ADD_F32 only): the tensors ``gemm_add_scratch`` asks for (float32, int32
-    zeros); the bits do not depend on it."""
-    _need(x, torch.bfloat16, "x")
+    zeros); the bits do not depend on it.  ``x`` may be a column slice of a wider matrix that starts at a multiple of 8
+    elements, and with a 32-bit store ``out`` may be a column slice too."""
+    _need_strided(x, torch.bfloat16, "x")
     _need(w, torch.bfloat16, "weight")
     if w.dim() != 2:
         raise ValueError("gemm_bf16: weight must be [N, K]")
@@ -448,7 +452,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows: int, ep
             raise ValueError("gemm_bf16: SwiGLU needs a stacked weight with an even number of rows")
         N //= 2
     want = torch.bfloat16 if epilogue in (EPI_BF16, EPI_SWIGLU_BF16) else torch.float32
-    _need(out, want, "out")
+    if epilogue == EPI_F32:
+        _need_strided(out, want, "out")
+    else:
+        _need(out, want, "out")
     if x.shape[1] != K or out.shape[1] != N or x.shape[0] < rows or out.shape[0] < rows:
         raise ValueError(f"gemm_bf16: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not match")
     if K % 8:
@@ -765,7 +772,7 @@ def gemm_qkv_rope_bf16(x: torch.Tensor, w_qkv: torch.Tensor, q_out: torch.Tensor
 
 # ------------------------------------------------------------------------------ mixers with a state per request
 
-RECUR_DECAY_PER_CHANNEL, RECUR_SCALAR_GATES = 0, 1
+RECUR_DECAY_PER_CHANNEL, RECUR_SCALAR_GATES, RECUR_BONUS_DECAY, RECUR_FIXED_DECAY = 0, 1, 2, 3
 RECUR_MAX_DIM = 256          # key channels of a head that the recurrence keeps in a lane's registers
 GATE_SIGMOID, GATE_SILU = 0, 1
 ACT_SILU, ACT_GELU_TANH, ACT_CLAMPED_SWISH = 0, 1, 2
@@ -782,7 +789,8 @@ def norm_shift(x: torch.Tensor, weight: torch.Tensor, mix: torch.Tensor, state: 
                eps: float) -> None:
     """out[r] = h[r] + (h_prev[r] - h[r]) * mix with h = rmsnorm(x) * weight and h_prev the h of the request's token
     before (from ``state`` [slots, width] for a request's first row of the step, which then receives the h of
-    the request's last row).  All 32-bit; ``out`` in float32 or bfloat16."""
+    the request's last row).  ``mix`` [width], or [n, width] for n shifted copies side by side in ``out`` [rows, n*width].
+    All 32-bit; ``out`` in float32 or bfloat16."""
     _need(x, torch.float32, "x")
     _need(weight, torch.float32, "norm weight")
     _need(mix, torch.float32, "mix")
@@ -790,24 +798,29 @@ def norm_shift(x: torch.Tensor, weight: torch.Tensor, mix: torch.Tensor, state: 
     for t, what in ((positions, "positions"), (row_seq, "row_seq"), (seq_rows, "seq_rows"), (slots, "slots")):
         _need(t, torch.int32, what)
     dim = x.shape[1]
-    if weight.numel() != dim or mix.numel() != dim or state.dim() != 2 or state.shape[1] < dim:
+    nmix = mix.numel() // max(dim, 1)
+    if weight.numel() != dim or nmix < 1 or mix.numel() != nmix * dim or state.dim() != 2 or state.shape[1] < dim:
         raise ValueError("norm_shift: weight, mix or state do not fit the rows' width")
-    if x.shape[0] < rows or out.shape[0] < rows or out.shape[1] != dim or positions.numel() < rows or row_seq.numel() < rows:
+    if x.shape[0] < rows or out.shape[0] < rows or out.shape[1] != nmix * dim or positions.numel() < rows or row_seq.numel() < rows:
         raise ValueError("norm_shift: buffers shorter than the rows")
     _check(_fn("bw_norm_shift")(x.data_ptr(), x.stride(0), weight.data_ptr(), mix.data_ptr(), state.data_ptr(), state.stride(0),
                                 positions.data_ptr(), row_seq.data_ptr(), seq_rows.data_ptr(), slots.data_ptr(),
-                                out.data_ptr(), _act_out(out, "out"), out.stride(0), rows, dim, float(eps), _stream()),
+                                out.data_ptr(), _act_out(out, "out"), out.stride(0), rows, dim, float(eps), nmix, _stream()),
            "norm_shift")
 
 
-def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gate: torch.Tensor, gate_off: int,
+def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, gate: Optional[torch.Tensor], gate_off: int,
                       gate2_off: int, bias: torch.Tensor, bias2: Optional[torch.Tensor], param: float, qscale: float,
                       state: torch.Tensor, out: torch.Tensor, seq_rows: torch.Tensor, slots: torch.Tensor,
-                      positions: torch.Tensor, nseq: int, heads: int, dim: int, vdim: int, scan=None) -> None:
+                      positions: torch.Tensor, nseq: int, heads: int, dim: int, vdim: int, scan=None, kscale: float = 1.0) -> None:
     """The recurrence S <- decay * S + k v^T, o = S^T (q * qscale) per head over every request's rows in order, from and
     to ``state`` [slots, elements].  RECUR_DECAY_PER_CHANNEL: decay = exp(logsigmoid(gate + bias) * param) per key
     channel (``gate`` [rows, >= gate_off + heads*dim]).  RECUR_SCALAR_GATES: capped input and forget gates per head
     (columns gate_off + h and gate2_off + h of ``gate``), a normaliser and a running maximum in the state; param = cap.
+    RECUR_BONUS_DECAY: decay = exp(-exp(gate + bias)) per key channel, and the read-out comes before the update:
+    o = (S + diag(bias2) k v^T)^T q with the S the token before left (``bias2`` [heads*dim]: the weight of the token's own
+    k v^T), then S <- decay * S + k v^T.  RECUR_FIXED_DECAY: one constant decay a head (``bias`` [heads]; ``gate`` None).
+    k is multiplied by ``kscale``.  ``state`` may be a column slice of a wider tensor.
 
     ``scan`` = (chunks [n, 4] int32 = (first row, rows, request, 1 if the request's last chunk), n, spans [k, 3] int32 =
     (request, its first chunk, its chunks), k, local, start): long portions run in three passes over their chunks (each
@@ -815,9 +828,10 @@ def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_o
     ``local`` and ``start`` float32 of n * heads * (dim*vdim + dim + 2) elements each; ``seq_rows`` then carries no rows
     for those requests (nseq may be 0).  The result differs from the one-pass order by the rounding of the walk's sums."""
     _need(proj, torch.float32, "proj")
-    _need(gate, torch.float32, "gate")
+    if mode != RECUR_FIXED_DECAY:
+        _need(gate, torch.float32, "gate")
     _need(bias, torch.float32, "bias")
-    _need(state, torch.float32, "state")
+    _need_strided(state, torch.float32, "state")
     _need(out, torch.float32, "out")
     for t, what in ((positions, "positions"), (seq_rows, "seq_rows"), (slots, "slots")):
         _need(t, torch.int32, what)
@@ -830,7 +844,17 @@ def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_o
         if bias.numel() != heads or bias2.numel() != heads or max(gate_off, gate2_off) + heads > gate.shape[1]:
             raise ValueError("linear_recurrence: gates or biases do not fit the heads")
         need = heads * (dim * vdim + dim + 1)
+    elif mode == RECUR_FIXED_DECAY:
+        if bias.numel() != heads:
+            raise ValueError("linear_recurrence: a constant decay a head is needed")
+        need = heads * dim * vdim
     else:
+        if mode == RECUR_BONUS_DECAY:
+            if bias2 is None:
+                raise ValueError("linear_recurrence: the read-out before the update needs the weights of the token's own k v^T")
+            _need(bias2, torch.float32, "bias2")
+            if bias2.numel() != heads * dim:
+                raise ValueError("linear_recurrence: the weights of the token's own k v^T do not fit heads x dim")
         if bias.numel() != heads * dim or gate_off + heads * dim > gate.shape[1]:
             raise ValueError("linear_recurrence: decay logits or bias do not fit heads x dim")
         need = heads * dim * vdim
@@ -850,15 +874,64 @@ def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_o
         _need(start, torch.float32, "scan records")
         if chunks.numel() < 4 * nchunks or spans.numel() < 3 * nspans or start.numel() < local.numel():
             raise ValueError("linear_recurrence: the scan's tables or records do not fit")
-    _check(_fn("bw_linear_recurrence")(int(mode), proj.data_ptr(), proj.stride(0), q_off, k_off, v_off, gate.data_ptr(),
-                                       gate.stride(0), gate_off, gate2_off, bias.data_ptr(),
-                                       0 if bias2 is None else bias2.data_ptr(), float(param), float(qscale), state.data_ptr(),
+    _check(_fn("bw_linear_recurrence")(int(mode), proj.data_ptr(), proj.stride(0), q_off, k_off, v_off,
+                                       0 if gate is None else gate.data_ptr(), 0 if gate is None else gate.stride(0),
+                                       gate_off, gate2_off, bias.data_ptr(),
+                                       0 if bias2 is None else bias2.data_ptr(), float(param), float(qscale), float(kscale), state.data_ptr(),
                                        state.stride(0), out.data_ptr(), out.stride(0), seq_rows.data_ptr(), slots.data_ptr(),
                                        positions.data_ptr(), nseq, heads, dim, vdim,
                                        0 if chunks is None else chunks.data_ptr(), nchunks,
                                        0 if spans is None else spans.data_ptr(), nspans,
                                        0 if local is None else local.data_ptr(), 0 if start is None else start.data_ptr(),
                                        0 if local is None else local.numel(), _stream()), "linear_recurrence")
+
+
+def rotate_halves_rows(x: torch.Tensor, offsets: Sequence[int], heads: int, dim: int, rot: int, cos: torch.Tensor,
+                       sin: torch.Tensor, positions: torch.Tensor, rows: int) -> None:
+    """One or two sections of ``x`` (float32 [rows, >= off + heads*dim], a section at each of ``offsets``) turned in place
+    by the rows' positions: of every head's first ``rot`` elements, element i is paired with element i + rot/2; the
+    tables are [positions, rot/2]."""
+    _need(x, torch.float32, "x")
+    _need(positions, torch.int32, "positions")
+    if rot == 0 or rows <= 0:
+        return
+    _need(cos, torch.float32, "cos table")
+    _need(sin, torch.float32, "sin table")
+    offs = [int(o) for o in offsets]
+    if not 1 <= len(offs) <= 2 or rot % 2 or rot > dim or cos.shape[1] != rot // 2 or sin.shape != cos.shape:
+        raise ValueError("rotate_halves_rows: one or two sections, tables [positions, rot/2], rot even and at most dim")
+    if x.shape[0] < rows or positions.numel() < rows or any(o < 0 or o + heads * dim > x.shape[1] for o in offs):
+        raise ValueError("rotate_halves_rows: the sections do not fit the rows")
+    _check(_fn("bw_rotate_halves_rows")(x.data_ptr(), x.stride(0), rows, heads, dim, rot, len(offs), offs[0], offs[-1], cos.data_ptr(),
+                                        sin.data_ptr(), positions.data_ptr(), _stream()), "rotate_halves_rows")
+
+
+def tanh_rows(x: torch.Tensor, rows: int) -> None:
+    """x[:rows] = tanh(x[:rows]) in place; ``x`` float32, a column slice will do."""
+    _need_strided(x, torch.float32, "x")
+    if x.shape[0] < rows:
+        raise ValueError("tanh_rows: fewer rows than asked for")
+    _check(_fn("bw_tanh_rows")(x.data_ptr(), x.stride(0), rows, x.shape[1], _stream()), "tanh_rows")
+
+
+def norm_mean(ys: Sequence[torch.Tensor], weights: Sequence[torch.Tensor], out: torch.Tensor, rows: int, eps: float) -> None:
+    """out[r] = mean over b of ys[b][r] / sqrt(mean(ys[b][r]^2) + eps) * weights[b], all 32-bit: up to four matrices of one
+    width, each normed row by row with a weight vector of its own."""
+    n = len(ys)
+    _need(out, torch.float32, "out")
+    dim = out.shape[1]
+    if not 1 <= n <= 4 or len(weights) != n or out.shape[0] < rows:
+        raise ValueError("norm_mean: one to four inputs, a weight vector each")
+    for y, w in zip(ys, weights):
+        _need_strided(y, torch.float32, "input")
+        _need(w, torch.float32, "weight")
+        if y.shape[1] != dim or y.shape[0] < rows or w.numel() != dim:
+            raise ValueError("norm_mean: inputs and weights must have out's width")
+    yp = (c_void_p * n)(*[y.data_ptr() for y in ys])
+    wp = (c_void_p * n)(*[w.data_ptr() for w in weights])
+    ld = (c_int * n)(*[y.stride(0) for y in ys])
+    _check(_fn("bw_norm_mean")(ctypes.cast(yp, c_void_p), ctypes.cast(ld, c_void_p), ctypes.cast(wp, c_void_p), n, out.data_ptr(),
+                               out.stride(0), rows, dim, float(eps), _stream()), "norm_mean")
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, per_head_weight: bool, g: torch.Tensor, g_off: int, gate: int,
@@ -1081,9 +1154,12 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
 def pair_rope_unit(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
                    cos: torch.Tensor, sin: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
                    v_cache: Optional[torch.Tensor], rows: int, heads: int, kv_heads: int, dim: int, vdim: int, head_size: int,
-                   rot: int, page_size: int, unit_norm: bool, eps: float, has_kv: bool, write_cache: bool) -> None:
-    """``src`` [rows, >= heads*dim (+ kv_heads*(dim+vdim))] float32: query heads, then key heads, then value heads.  The
-    first ``rot`` elements of every query and key head are rotated pair by pair ((2i, 2i+1) by the angle of table
+                   rot: int, page_size: int, unit_norm: bool, eps: float, has_kv: bool, write_cache: bool,
+                   halves: bool = False, values_are_keys: bool = False) -> None:
+    """``src`` [rows, >= heads*dim (+ kv_heads*(dim+vdim))] float32: query heads, then key heads, then value heads (with
+    ``values_are_keys`` no value heads: a value head is its key head as projected, before rotation).  The
+    first ``rot`` elements of every query and key head are rotated pair by pair ((2i, 2i+1), or with ``halves``
+    (i, i + rot/2), by the angle of table
     column i at the row's position), the head is then divided by its root mean square if ``unit_norm``; queries go to
     ``q_out`` [rows, heads*head_size], keys and values (as they are) into the row's page slot, all padded with zeros
     to ``head_size``.  Page layouts: bfloat16 keys [kv head][slot][element], values [kv head][element][slot]; float32
@@ -1095,7 +1171,9 @@ def pair_rope_unit(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Te
     _need(cos, torch.float32, "cos table")
     _need(sin, torch.float32, "sin table")
     bf = _act_out(q_out, "q_out")
-    need = heads * dim + (kv_heads * (dim + vdim) if has_kv else 0)
+    need = heads * dim + (kv_heads * (dim + (0 if values_are_keys else vdim)) if has_kv else 0)
+    if values_are_keys and vdim != dim:
+        raise ValueError("pair_rope_unit: values that are the keys have the keys' size")
     if src.shape[1] < need or src.shape[0] < rows or q_out.shape[0] < rows or q_out.shape[1] != heads * head_size:
         raise ValueError("pair_rope_unit: src or q_out do not fit")
     if positions.numel() < rows or row_seq.numel() < rows:
@@ -1114,7 +1192,8 @@ def pair_rope_unit(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Te
     _check(_fn("bw_pair_rope_unit")(src.data_ptr(), src.stride(0), positions.data_ptr(), row_seq.data_ptr(), block_table.data_ptr(),
                                     block_table.stride(0), cos.data_ptr(), sin.data_ptr(), q_out.data_ptr(), kp, vp, bf, rows,
                                     heads, kv_heads, dim, vdim, head_size, rot, page_size, int(unit_norm), float(eps),
-                                    int(has_kv), int(write_cache and has_kv), _stream()), "pair_rope_unit")
+                                    int(has_kv), int(write_cache and has_kv), int(halves), int(values_are_keys), _stream()),
+           "pair_rope_unit")
 
 
 def whole_norm_kv(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Tensor, block_table: torch.Tensor,
@@ -1162,16 +1241,18 @@ def whole_norm_kv(src: torch.Tensor, positions: torch.Tensor, row_seq: torch.Ten
                                    page_size, int(bool(write_cache)), _stream()), "whole_norm_kv")
 
 
-def gate_mul(av: torch.Tensor, head_size: int, g: torch.Tensor, out: torch.Tensor, rows: int, heads: int, vdim: int) -> None:
-    """out[r, h*vdim + d] = av[r, h*head_size + d] * sigmoid(g[r, h*vdim + d]); ``g`` float32 (a column slice will do)."""
-    if g.dtype != torch.float32 or g.stride(1) != 1 or g.shape[1] < heads * vdim:
-        raise ValueError("gate_mul: g must be float32 with contiguous rows of heads*vdim")
+def gate_mul(av: torch.Tensor, head_size: int, g: torch.Tensor, out: torch.Tensor, rows: int, heads: int, vdim: int,
+             per_head: bool = False) -> None:
+    """out[r, h*vdim + d] = av[r, h*head_size + d] * sigmoid(g[r, h*vdim + d]), or with ``per_head`` * sigmoid(g[r, h]);
+    ``g`` float32 (a column slice will do)."""
+    if g.dtype != torch.float32 or g.stride(1) != 1 or g.shape[1] < (heads if per_head else heads * vdim):
+        raise ValueError("gate_mul: g must be float32 with contiguous rows of heads*vdim (a gate a head: of heads)")
     if av.shape[1] != heads * head_size or out.shape[1] != heads * vdim or vdim > head_size:
         raise ValueError("gate_mul: av or out do not fit")
     if min(av.shape[0], out.shape[0], g.shape[0]) < rows:
         raise ValueError("gate_mul: buffers shorter than the rows")
     _check(_fn("bw_gate_mul")(av.data_ptr(), _act_out(av, "av"), av.stride(0), head_size, g.data_ptr(), g.stride(0), out.data_ptr(),
-                              _act_out(out, "out"), out.stride(0), rows, heads, vdim, _stream()), "gate_mul")
+                              _act_out(out, "out"), out.stride(0), rows, heads, vdim, int(per_head), _stream()), "gate_mul")
 
 
 def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: torch.Tensor, ri_bias: torch.Tensor,
@@ -1208,8 +1289,9 @@ def rglru_scan(y: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, ra_bias: t
 
 
 def norm_add(y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rows: int, eps: float,
-             rounded: Optional[torch.Tensor] = None, combine: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None) -> None:
-    """x[:rows] += y / sqrt(mean(y^2) + eps) * weight, all 32-bit.  ``rounded`` (bfloat16, x's shape): also receives the new
+             rounded: Optional[torch.Tensor] = None, combine: Optional[Tuple[torch.Tensor, torch.Tensor, int]] = None,
+             scale: float = 1.0) -> None:
+    """x[:rows] += scale * (y / sqrt(mean(y^2) + eps) * weight), all 32-bit.  ``rounded`` (bfloat16, x's shape): also receives the new
     rows rounded, for products that follow.  ``combine`` = (place, wts, top): row r of the normed operand is
     sum_j wts[r, j] * y[place[r*top + j]] (j ascending, the chain of ``moe_combine``) instead of y[r]."""
     _need(y, torch.float32, "y")
@@ -1232,7 +1314,7 @@ def norm_add(y: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, rows: int, 
     _check(_fn("bw_norm_add")(y.data_ptr(), y.stride(0), weight.data_ptr(), _is_bf16(weight, "weight"), x.data_ptr(), x.stride(0),
                               0 if rounded is None else rounded.data_ptr(), 0 if rounded is None else rounded.stride(0),
                               rows, dim, float(eps), 0 if place is None else place.data_ptr(), 0 if wts is None else wts.data_ptr(),
-                              int(top), _stream()), "norm_add")
+                              int(top), float(scale), _stream()), "norm_add")
 
 
 def softcap(x: torch.Tensor, rows: int, cap: float) -> None:
@@ -1258,11 +1340,26 @@ def moe_max_tiles(slots: int, experts: int) -> int:
     return int(_fn("bw_moe_max_tiles")(int(slots), int(experts)))
 
 
+SCORE_SOFTMAX, SCORE_SIGMOID = 0, 1
+
+
+def _route_rule(score: int, correction: Optional[torch.Tensor], group_best: int, experts: int):
+    if score not in (SCORE_SOFTMAX, SCORE_SIGMOID) or not 1 <= int(group_best) <= 4:
+        raise ValueError("moe_route: scores are a softmax or sigmoids; a group's score sums one to four of its best")
+    if correction is not None:
+        _need(correction, torch.float32, "correction")
+        if correction.numel() != experts:
+            raise ValueError("moe_route: a correction per expert is needed")
+    return int(score), 0 if correction is None else correction.data_ptr(), int(group_best)
+
+
 def moe_route(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor,
-              weight_scale: float = 1.0, experts: Optional[int] = None) -> None:
-    """Per row: softmax over the experts' logits; the ``top`` best experts among those of the ``keep`` best of ``groups``
-    equal groups of neighbours (a group's score: its best expert's); ``ids`` [rows, top] int32 in the order chosen,
-    ``wts`` [rows, top] their scores."""
+              weight_scale: float = 1.0, experts: Optional[int] = None, score: int = SCORE_SOFTMAX,
+              correction: Optional[torch.Tensor] = None, group_best: int = 1) -> None:
+    """Per row: scores = softmax over the experts' logits (``score`` SCORE_SIGMOID: the sigmoid of each); the ``top`` best
+    experts among those of the ``keep`` best of ``groups`` equal groups of neighbours, judged by score + ``correction``
+    (a group's score: the sum of its ``group_best`` best); ``ids`` [rows, top] int32 in the order chosen,
+    ``wts`` [rows, top] their scores (without the correction)."""
     _need(logits, torch.float32, "logits")
     _need(ids, torch.int32, "ids")
     _need(wts, torch.float32, "wts")
@@ -1272,7 +1369,8 @@ def moe_route(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int,
     if experts % groups or not 1 <= keep <= groups or not 1 <= top <= keep * (experts // groups):
         raise ValueError("moe_route: groups, keep and top do not fit the experts")
     _check(_fn("bw_moe_route")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, float(weight_scale),
-                               ids.data_ptr(), wts.data_ptr(), _stream()), "moe_route")
+                               *_route_rule(score, correction, group_best, experts), ids.data_ptr(), wts.data_ptr(), _stream()),
+           "moe_route")
 
 
 def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor,
@@ -1288,7 +1386,8 @@ def moe_plan(ids: torch.Tensor, slots: int, experts: int, sorted_slots: torch.Te
 
 def moe_route_plan(logits: torch.Tensor, rows: int, top: int, groups: int, keep: int, ids: torch.Tensor, wts: torch.Tensor,
                    sorted_slots: torch.Tensor, place: torch.Tensor, tiles: torch.Tensor, meta: torch.Tensor,
-                   weight_scale: float = 1.0, experts: Optional[int] = None) -> None:
+                   weight_scale: float = 1.0, experts: Optional[int] = None, score: int = SCORE_SOFTMAX,
+                   correction: Optional[torch.Tensor] = None, group_best: int = 1) -> None:
     """``moe_route`` followed by ``moe_plan`` over the rows' choices; steps of up to 16 rows do both in one launch.
     ``weight_scale``: the chosen scores are multiplied by it; ``experts``: the leading columns of ``logits`` that are the
     experts' (all of them by default)."""
@@ -1304,7 +1403,7 @@ def moe_route_plan(logits: torch.Tensor, rows: int, top: int, groups: int, keep:
     if tiles.numel() < 4 * moe_max_tiles(slots, experts) or meta.numel() < 1:
         raise ValueError("moe_route_plan: the plan's tables are too small")
     _check(_fn("bw_moe_route_plan")(logits.data_ptr(), logits.stride(0), rows, experts, top, groups, keep, float(weight_scale),
-                                    ids.data_ptr(), wts.data_ptr(),
+                                    *_route_rule(score, correction, group_best, experts), ids.data_ptr(), wts.data_ptr(),
                                     sorted_slots.data_ptr(), place.data_ptr(), tiles.data_ptr(), meta.data_ptr(), _stream()),
            "moe_route_plan")
 

@@ -38,7 +38,8 @@ __device__ __forceinline__ float row_sumsq(const float* __restrict__ xr, int dim
 
 // ------------------------------------------------------------------------- RMSNorm + token shift
 
-// out[r] = h[r] + (h'[r] - h[r]) * mix with h = (x * inv_rms) * w and h' the h of the request's previous token: the
+// out[r][m] = h[r] + (h'[r] - h[r]) * mix[m] for each of nmix mixing vectors (out rows hold nmix blocks of dim elements), with
+// h = (x * inv_rms) * w and h' the h of the request's previous token: the
 // row above, or for the first row of a request in this step what the state slot holds (zeros for a new request).
 // The wave of a request's first row also leaves the h of the request's last row in the slot, after it has read it:
 // nothing else reads or writes that slot in this launch.  A wave a row.
@@ -49,7 +50,7 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
                                                          const int32_t* __restrict__ row_seq,
                                                          const int32_t* __restrict__ seq_rows,
                                                          const int32_t* __restrict__ slots, OT* __restrict__ out, int ldo,
-                                                         int rows, int dim, float eps) {
+                                                         int rows, int dim, float eps, int nmix) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * (blockDim.x >> 6) + wave_index();
   if (row >= rows) return;
@@ -91,18 +92,25 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
       for (int jj = 0; jj < UN; ++jj) {
         const int c = c0 + 64 * jj + lane;
         if (c >= nvec) continue;
-        f32x4 r, keep;
+        f32x4 hq, dq, keep;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float h = (xq[jj][e] * inv) * wq[jj][e];
+          hq[e] = (xq[jj][e] * inv) * wq[jj][e];
           const float hp = is_first ? pq[jj][e] : (pq[jj][e] * invp) * wq[jj][e];
-          r[e] = fmaf(hp - h, mq[jj][e], h);
+          dq[e] = hp - hq[e];
           keep[e] = (lq[jj][e] * invl) * wq[jj][e];
         }
-        if constexpr (sizeof(OT) == 2) {
-          *reinterpret_cast<u32x2*>(o + 4 * c) = (u32x2){pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
-        } else {
-          *reinterpret_cast<f32x4*>(o + 4 * c) = r;
+        for (int m = 0; m < nmix; ++m) {
+          const f32x4 mm = m == 0 ? mq[jj] : mv[(size_t)m * nvec + c];
+          f32x4 r;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r[e] = fmaf(dq[e], mm[e], hq[e]);
+          OT* om = o + (size_t)m * dim;
+          if constexpr (sizeof(OT) == 2) {
+            *reinterpret_cast<u32x2*>(om + 4 * c) = (u32x2){pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+          } else {
+            *reinterpret_cast<f32x4*>(om + 4 * c) = r;
+          }
         }
         if (is_first) reinterpret_cast<f32x4*>(st)[c] = keep;
       }
@@ -116,7 +124,7 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
     for (int i = lane; i < dim; i += 64) {
       const float h = (xr[i] * inv) * w[i];
       const float hp = (xp[i] * invp) * w[i];
-      store_act(o + i, fmaf(hp - h, mix[i], h));
+      for (int m = 0; m < nmix; ++m) store_act(o + (size_t)m * dim + i, fmaf(hp - h, mix[(size_t)m * dim + i], h));
     }
     return;
   }
@@ -126,14 +134,14 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
   for (int i = lane; i < dim; i += 64) {
     const float h = (xr[i] * inv) * w[i];
     const float hp = st[i];
-    store_act(o + i, fmaf(hp - h, mix[i], h));
+    for (int m = 0; m < nmix; ++m) store_act(o + (size_t)m * dim + i, fmaf(hp - h, mix[(size_t)m * dim + i], h));
     st[i] = (xl[i] * invl) * w[i];
   }
 }
 
 // ------------------------------------------------------------------------- the linear recurrence
 
-enum { RECUR_DECAY_PER_CHANNEL = 0, RECUR_SCALAR_GATES = 1 };
+enum { RECUR_DECAY_PER_CHANNEL = 0, RECUR_SCALAR_GATES = 1, RECUR_BONUS_DECAY = 2, RECUR_FIXED_DECAY = 3 };
 
 // The sum over the lanes l, l + 64/SPLIT, ... that hold the parts of one column (every one of them gets it).
 template <int SPLIT>
@@ -158,7 +166,7 @@ struct RecurArgs {
   const float* bias;       // per channel: [heads*dim]; scalar gates: input-gate bias [heads]
   const float* bias2;      // scalar gates: forget-gate bias [heads]
   float param;             // per channel: 1 / tau; scalar gates: the cap
-  float qscale;
+  float qscale, kscale;
   float* state;            // [slots, state_ld]: S [heads][dim][vdim]; scalar gates also n [heads][dim] and m [heads]
   long long state_ld;
   float* out;              // [rows, ldo]: head h at columns h*vdim ..
@@ -185,6 +193,11 @@ struct RecurArgs {
 //   n is spread over the lanes (lane l holds n[l], n[l+64], ...); every wave of a head computes it, the wave of
 //   column block 0 stores it.
 //
+// RECUR_BONUS_DECAY:  alpha[d] = exp(-exp(z[d] + bias[d]));  o[j] = sum_d (S[d][j] + u[d] k[d] v[j]) q[d] with the S of the token
+//   before (the token's own k v^T is read through the bonus u = bias2 [heads*dim]), then S[d][j] <- alpha[d] S[d][j] + k[d] v[j].
+// RECUR_FIXED_DECAY:  as per channel with one constant decay a head, alpha[d] = bias[head]; no logits are read.
+// (q is multiplied by qscale and k by kscale on their way into LDS.)
+//
 // A request's long portion can also run in three passes over chunks of its rows, which gives every chunk waves of its
 // own: PHASE 1 runs every chunk from a zero state (no read-out) and leaves the chunk's own contribution and its decay;
 // recurrence_scan_kernel walks a request's chunks in order and leaves the state each one starts from; PHASE 3 runs every
@@ -195,6 +208,7 @@ struct RecurArgs {
 template <int MODE, int DPAD, int PHASE>
 __global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a) {
   constexpr bool GATES = MODE == RECUR_SCALAR_GATES;
+  constexpr bool BONUS = MODE == RECUR_BONUS_DECAY, FIXED = MODE == RECUR_FIXED_DECAY;
   constexpr int NN = (DPAD + 63) / 64;
   constexpr bool READ_OUT = PHASE != 1;
   // A column's key channels are split over SPLIT lanes (lane l, l + COLS, ... hold consecutive parts of column l mod COLS): a
@@ -208,6 +222,7 @@ __global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a)
   __shared__ float as[GATES ? 1 : RC][GATES ? 1 : DPAD];
   __shared__ float gi[RC], gf[RC];
   __shared__ float vs[RW][RC][64];
+  __shared__ float us[BONUS ? DPAD : 1];
   const int lane = threadIdx.x & 63, wv = wave_index();
   const int cb = blockIdx.x * RW + wv, h = blockIdx.y;
   const int dim = a.dim, vdim = a.vdim;
@@ -259,6 +274,10 @@ __global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a)
     for (int i = 0; i < NN; ++i) nreg[i] = 1.0f;
   }
 
+  if constexpr (BONUS) {
+    for (int d = threadIdx.x; d < DPAD; d += 64 * RW) us[d] = d < dim ? a.bias2[h * dim + d] : 0.0f;
+  }
+  const float fixed_decay = FIXED ? a.bias[h] : 0.0f;
   for (int t0 = 0; t0 < count; t0 += RC) {
     const int tc = min(RC, count - t0);
     __syncthreads();
@@ -274,7 +293,7 @@ __global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a)
         const float* pr = a.proj + row * a.ldp;
         qv[u] = in ? pr[a.q_off + h * dim + d] : 0.0f;
         kv[u] = in ? pr[a.k_off + h * dim + d] : 0.0f;
-        if constexpr (!GATES) zv[u] = in ? a.gate[row * a.ldg + a.gate_off + h * dim + d] + a.bias[h * dim + d] : 0.0f;
+        if constexpr (!GATES && !FIXED) zv[u] = in ? a.gate[row * a.ldg + a.gate_off + h * dim + d] + a.bias[h * dim + d] : 0.0f;
       }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -282,8 +301,10 @@ __global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a)
         if (e >= tc * DPAD) continue;
         const int t = e / DPAD, d = e % DPAD;
         qs[t][d] = qv[u] * a.qscale;
-        ks[t][d] = kv[u];
-        if constexpr (!GATES) as[t][d] = d < dim ? bw_expf(log_sigmoid(zv[u]) * a.param) : 0.0f;
+        ks[t][d] = kv[u] * a.kscale;
+        if constexpr (FIXED) as[t][d] = d < dim ? fixed_decay : 0.0f;
+        else if constexpr (BONUS) as[t][d] = d < dim ? bw_expf(-bw_expf(zv[u])) : 0.0f;
+        else if constexpr (!GATES) as[t][d] = d < dim ? bw_expf(log_sigmoid(zv[u]) * a.param) : 0.0f;
       }
     }
     if constexpr (GATES) {
@@ -307,8 +328,14 @@ __global__ __launch_bounds__(64 * RW) void linear_recurrence_kernel(RecurArgs a)
         const float v = vs[wv][t][col];
 #pragma unroll
         for (int d = 0; d < DH; ++d) {
-          Sreg[d] = fmaf(as[t][dbase + d], Sreg[d], ks[t][dbase + d] * v);
-          if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][dbase + d], o);
+          if constexpr (BONUS) {
+            const float kv = ks[t][dbase + d] * v;
+            if constexpr (READ_OUT) o = fmaf(fmaf(us[dbase + d], kv, Sreg[d]), qs[t][dbase + d], o);
+            Sreg[d] = fmaf(as[t][dbase + d], Sreg[d], kv);
+          } else {
+            Sreg[d] = fmaf(as[t][dbase + d], Sreg[d], ks[t][dbase + d] * v);
+            if constexpr (READ_OUT) o = fmaf(Sreg[d], qs[t][dbase + d], o);
+          }
         }
         if constexpr (PHASE == 1) {
 #pragma unroll
@@ -495,28 +522,70 @@ __global__ void glu_kernel(const float* __restrict__ gu, int ldg, OT* __restrict
   store_act(hout + idx, h);
 }
 
+
+// ------------------------------------------------------------------------- rotation of 32-bit projections in place
+
+// Sections of a row of 32-bit projections ([heads][dim] each, at columns off[s]) turned in place by the row's position:
+// of every head's first rot elements, element i < rot/2 is paired with element i + rot/2, (u, v) -> (u c - v s, v c + u s)
+// with c, s from the tables' row of the position.  A thread a pair.
+struct RotateRowsArgs {
+  float* x;
+  int ldx, rows, heads, dim, rot, sections;
+  int off[2];
+  const float* cos_table;     // [positions, rot / 2]
+  const float* sin_table;
+  const int32_t* positions;
+};
+
+__global__ __launch_bounds__(256) void rotate_halves_rows_kernel(RotateRowsArgs a) {
+  const int half = a.rot / 2;
+  const int per_row = a.sections * a.heads * half;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)a.rows * per_row) return;
+  const int row = (int)(idx / per_row);
+  int r = (int)(idx % per_row);
+  const int sec = r / (a.heads * half);
+  r %= a.heads * half;
+  const int h = r / half, i = r % half;
+  const int pos = a.positions[row];
+  if (pos < 0) return;
+  float* p = a.x + (size_t)row * a.ldx + a.off[sec] + (size_t)h * a.dim;
+  const float c = a.cos_table[(size_t)pos * half + i], s = a.sin_table[(size_t)pos * half + i];
+  const float u = p[i], v = p[i + half];
+  p[i] = u * c - v * s;
+  p[i + half] = v * c + u * s;
+}
+
+// x <- tanh(x) over [rows, cols] of 32-bit values
+__global__ __launch_bounds__(256) void tanh_rows_kernel(float* __restrict__ x, int ld, int rows, int cols) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)rows * cols) return;
+  float* p = x + (idx / cols) * ld + (idx % cols);
+  *p = tanhf(*p);
+}
+
 }  // namespace
 
 extern "C" int bw_norm_shift(const float* x, int ldx, const float* w, const float* mix, float* state, long long state_ld,
                              const int32_t* positions, const int32_t* row_seq, const int32_t* seq_rows,
                              const int32_t* slots, void* out, int out_is_bf16, int ldo, int rows, int dim, float eps,
-                             void* stream) {
+                             int nmix, void* stream) {
   if (rows <= 0) return 0;
-  if (dim <= 0 || ldx < dim || ldo < dim || state_ld < dim) return -2;
+  if (dim <= 0 || nmix < 1 || ldx < dim || (long long)ldo < (long long)nmix * dim || state_ld < dim) return -2;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((rows + 3) / 4), block(256);
   if (out_is_bf16)
     hipLaunchKernelGGL(norm_shift_kernel<bf16_t>, grid, block, 0, s, x, ldx, w, mix, state, state_ld, positions, row_seq,
-                       seq_rows, slots, (bf16_t*)out, ldo, rows, dim, eps);
+                       seq_rows, slots, (bf16_t*)out, ldo, rows, dim, eps, nmix);
   else
     hipLaunchKernelGGL(norm_shift_kernel<float>, grid, block, 0, s, x, ldx, w, mix, state, state_ld, positions, row_seq,
-                       seq_rows, slots, (float*)out, ldo, rows, dim, eps);
+                       seq_rows, slots, (float*)out, ldo, rows, dim, eps, nmix);
   return BW_LAUNCH_CHECK();
 }
 
 extern "C" int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_off, int k_off, int v_off, const float* gate,
                                     int ldg, int gate_off, int gate2_off, const float* bias, const float* bias2, float param,
-                                    float qscale, float* state, long long state_ld, float* out, int ldo,
+                                    float qscale, float kscale, float* state, long long state_ld, float* out, int ldo,
                                     const int32_t* seq_rows, const int32_t* slots, const int32_t* positions, int nseq,
                                     int heads, int dim, int vdim, const int32_t* chunks, int nchunks, const int32_t* spans,
                                     int nspans, float* scan_local, float* scan_start, long long scan_floats, void* stream) {
@@ -528,11 +597,15 @@ extern "C" int bw_linear_recurrence(int mode, const float* proj, int ldp, int q_
   if (heads <= 0 || dim <= 0 || vdim <= 0 || ldo < heads * vdim) return -2;
   const long long need = (long long)heads * dim * vdim + (mode == RECUR_SCALAR_GATES ? (long long)heads * dim + heads : 0);
   if (state_ld < need) return -2;
-  RecurArgs a{proj, ldp, q_off, k_off, v_off, gate, ldg, gate_off, gate2_off, bias, bias2, param, qscale, state, state_ld,
+  if (bias == nullptr || (mode != RECUR_FIXED_DECAY && gate == nullptr) || ((mode == RECUR_SCALAR_GATES || mode == RECUR_BONUS_DECAY) && bias2 == nullptr))
+    return -2;
+  RecurArgs a{proj, ldp, q_off, k_off, v_off, gate, ldg, gate_off, gate2_off, bias, bias2, param, qscale, kscale, state, state_ld,
               out, ldo, seq_rows, slots, positions, heads, dim, vdim, chunks, scan_local, scan_start};
   hipStream_t s = (hipStream_t)stream;
   if (mode == RECUR_SCALAR_GATES) return launch_recurrence_passes<RECUR_SCALAR_GATES>(a, nseq, nchunks, spans, nspans, s);
   if (mode == RECUR_DECAY_PER_CHANNEL) return launch_recurrence_passes<RECUR_DECAY_PER_CHANNEL>(a, nseq, nchunks, spans, nspans, s);
+  if (mode == RECUR_BONUS_DECAY) return launch_recurrence_passes<RECUR_BONUS_DECAY>(a, nseq, nchunks, spans, nspans, s);
+  if (mode == RECUR_FIXED_DECAY) return launch_recurrence_passes<RECUR_FIXED_DECAY>(a, nseq, nchunks, spans, nspans, s);
   return -2;
 }
 
@@ -562,5 +635,24 @@ extern "C" int bw_glu(const float* gate_up, int ldg, void* h, int out_is_bf16, i
   const dim3 grid((unsigned)((n + 255) / 256)), block(256);
   if (out_is_bf16) hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, block, 0, s, gate_up, ldg, (bf16_t*)h, n, inter, act, limit, alpha, row_gate, ld_row_gate);
   else hipLaunchKernelGGL(glu_kernel<float>, grid, block, 0, s, gate_up, ldg, (float*)h, n, inter, act, limit, alpha, row_gate, ld_row_gate);
+  return BW_LAUNCH_CHECK();
+}
+
+extern "C" int bw_rotate_halves_rows(float* x, int ldx, int rows, int heads, int dim, int rot, int sections, int off0, int off1,
+                                     const float* cos_table, const float* sin_table, const int32_t* positions, void* stream) {
+  if (rows <= 0 || rot == 0) return 0;
+  if (heads <= 0 || dim <= 0 || rot < 0 || rot % 2 || rot > dim || sections < 1 || sections > 2) return -2;
+  if (off0 < 0 || off0 + heads * dim > ldx || (sections == 2 && (off1 < 0 || off1 + heads * dim > ldx))) return -2;
+  RotateRowsArgs a{x, ldx, rows, heads, dim, rot, sections, {off0, off1}, cos_table, sin_table, positions};
+  const long long n = (long long)rows * sections * heads * (rot / 2);
+  hipLaunchKernelGGL(rotate_halves_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, a);
+  return BW_LAUNCH_CHECK();
+}
+
+extern "C" int bw_tanh_rows(float* x, int ld, int rows, int cols, void* stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  if (ld < cols) return -2;
+  const long long n = (long long)rows * cols;
+  hipLaunchKernelGGL(tanh_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, ld, rows, cols);
   return BW_LAUNCH_CHECK();
 }

@@ -26,6 +26,7 @@ class CallBinding:
     group: int                       # -1: the mixer keeps no paged cache
     cache_index: int                 # index of the cache inside its group's storage
     writes_cache: bool
+    adds_embedding: bool = False     # the embedding's output is added to the stream right before this call
     k_cache: Optional[torch.Tensor] = None
     v_cache: Optional[torch.Tensor] = None
     state: Optional[torch.Tensor] = None
@@ -47,7 +48,7 @@ class AssembledModel:
                 if kind is None:
                     raise ValueError(f"block '{ls.block}' has no role '{role}'; its roles: {sorted(block_cls.roles)}")
                 parts[role] = lookup(base.KINDS[kind], kind.replace("_", "-"), ps.kind)(ps.params, runtime)
-            self.layers.append(block_cls(parts, runtime))
+            self.layers.append(block_cls(parts, runtime, ls.params) if ls.params else block_cls(parts, runtime))
         self.final_norm = lookup(base.NORMS, "norm", spec.final_norm.kind)(spec.final_norm.params, runtime)
         self.lm_head = lookup(base.HEADS, "head", spec.lm_head.kind)(spec.lm_head.params, runtime)
         self._plan_caches(spec.schedule)
@@ -113,7 +114,7 @@ class AssembledModel:
             bs = self.layers[c.layer].state_spec()
             if bs is not None:
                 self.block_state_specs[idx] = bs
-            self.calls.append(CallBinding(idx, c.layer, c.cache, group, cindex, c.writes_cache))
+            self.calls.append(CallBinding(idx, c.layer, c.cache, group, cindex, c.writes_cache, c.adds_embedding))
 
     # ------------------------------------------------------------------ tensors
     def _parts_with_prefix(self):
@@ -166,7 +167,13 @@ class AssembledModel:
         ws = ctx.ws
         ctx.forward_notes = {}           # what parts tell later parts within this pass (a rounded copy of the stream that is current)
         x = self.embedding.forward(ctx)
+        first = None
+        if any(call.adds_embedding for call in ctx.calls):
+            first = ws.buffer("embedding_output", self.spec.width, torch.float32)
+            ops.convert(x, first, ctx.rows)              # (a copy: the layers change x in place)
         for call in ctx.calls:
+            if call.adds_embedding:
+                ops.add_(x, first, ctx.rows)
             self.layers[call.layer].forward(ctx, call, x)
         count = ctx.num_wanted
         if count == 0:

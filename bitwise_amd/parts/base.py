@@ -46,6 +46,7 @@ class LayerSpec:
     """
     block: str                                         # arrangement of the parts, e.g. "prenorm"
     parts: Dict[str, PartSpec] = field(default_factory=dict)   # role -> part
+    params: Dict[str, Any] = field(default_factory=dict)       # constants of the arrangement itself
 
     @classmethod
     def prenorm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec, ffn_norm: PartSpec) -> "LayerSpec":
@@ -62,11 +63,15 @@ class LayerCall:
     """One entry of the schedule: run ``layer``, with cache number ``cache``.
 
     ``writes_cache`` False means the call only reads a cache that an earlier call of
-    the same step wrote (its own keys and values are not stored).
+    the same step wrote (its own keys and values are not stored).  ``adds_embedding``: the
+    embedding's output (the stream as it was before the first call) is added to the stream
+    right before this call: what a model does that runs some of its layers several times and
+    feeds the input in again at the start of every further pass.
     """
     layer: int
     cache: int
     writes_cache: bool = True
+    adds_embedding: bool = False
 
 
 @dataclass
@@ -254,6 +259,12 @@ class Mixer(Part):
         norm and ``forward`` one after the other.  The result must be the same bits."""
         return False
 
+    def forward_add_normed(self, ctx, call, h, norm, x) -> bool:
+        """Optional: x += norm(mixer(h)) with the norm behind the mixer riding in the mixer's last kernel.  Return False
+        (and do nothing) if this part or this norm cannot; the block then calls ``forward_out`` and the norm one after
+        the other.  The result must be the same bits."""
+        return False
+
 
 class FeedForward(Part):
     def forward_with_norm(self, ctx, x, norm, residual) -> bool:
@@ -286,8 +297,8 @@ class Block(Part):
     roles: Dict[str, str] = {}
     optional_roles: Tuple[str, ...] = ()      # roles a layer may leave out (the attribute is None then)
 
-    def __init__(self, parts: Dict[str, Part], runtime):
-        super().__init__({}, runtime)
+    def __init__(self, parts: Dict[str, Part], runtime, params: Optional[Dict[str, Any]] = None):
+        super().__init__(params or {}, runtime)
         missing = [r for r in self.roles if r not in parts and r not in self.optional_roles]
         extra = [r for r in parts if r not in self.roles]
         if missing or extra:

@@ -116,3 +116,42 @@ class PostNormBlock(Block):
             else:
                 self.feed_forward.forward_out(ctx, h, y)
                 self._add(ctx, self.ffn_norm, y, x)
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """x += norm1b(mixer(norm1(x))); x += norm2b(feed_forward(norm2(x))): a norm in front of each sublayer and another
+    behind it, on its way into the stream (a factor on that second norm, its ``scale``, weighs the sublayer against the
+    stream).  A layer may leave the feed-forward (and its two norms) out.  A mixer norm with state of its own (a token
+    shift) gets the call's ``block_state``."""
+
+    roles = {"mixer_norm": "norm", "mixer_post_norm": "norm", "ffn_norm": "norm", "ffn_post_norm": "norm", "mixer": "mixer",
+             "feed_forward": "feed_forward"}
+    optional_roles = ("ffn_norm", "ffn_post_norm", "feed_forward")
+    graph_safe = True
+    launches_through_ops = True
+
+    def __init__(self, parts, runtime, params=None):
+        super().__init__(parts, runtime, params)
+        if len({self.feed_forward is None, self.ffn_norm is None, self.ffn_post_norm is None}) != 1:
+            raise ValueError("sandwich block: a feed-forward and its two norms come together or not at all")
+
+    def state_spec(self):
+        return self.mixer_norm.state_spec()
+
+    def forward(self, ctx, call, x) -> None:
+        if call.block_state is not None:
+            h = self.mixer_norm.forward(ctx, x, state=call.block_state)
+        else:
+            h = self.mixer_norm.forward(ctx, x)
+        if not self.mixer.forward_add_normed(ctx, call, h, self.mixer_post_norm, x):
+            y = ctx.ws.buffer("sublayer_out", x.shape[1], torch.float32)
+            self.mixer.forward_out(ctx, call, h, y)
+            self.mixer_post_norm.add_normed(ctx, y, x)
+        if self.feed_forward is None:
+            return
+        h = self.ffn_norm.forward(ctx, x)
+        if not self.feed_forward.forward_add_normed(ctx, h, self.ffn_post_norm, x):
+            y = ctx.ws.buffer("sublayer_out", x.shape[1], torch.float32)
+            self.feed_forward.forward_out(ctx, h, y)
+            self.ffn_post_norm.add_normed(ctx, y, x)

@@ -13,7 +13,8 @@ from .linear import Linear
 
 @register_embedding("embedding")
 class TokenEmbedding(Embedding):
-    """params: vocab, width.  tensor: weight [vocab, width], gathered as 32-bit rows."""
+    """params: vocab, width; optional ``norm`` = {tensor, eps}: the gathered row is divided by its root mean square and
+    multiplied by that weight vector before it becomes the stream.  tensor: weight [vocab, width], gathered as 32-bit rows."""
 
     graph_safe = True
     launches_through_ops = True
@@ -23,12 +24,19 @@ class TokenEmbedding(Embedding):
         self.vocab, self.width = int(params["vocab"]), int(params["width"])
         self.tensor = str(params.get("tensor", "weight"))      # the table's name behind the prefix
         self.weight: Optional[torch.Tensor] = None
+        self.norm = dict(params["norm"]) if params.get("norm") else None
+        self.norm_weight: Optional[torch.Tensor] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
-        return {self.tensor: TensorSpec((self.vocab, self.width), "embedding")}
+        out = {self.tensor: TensorSpec((self.vocab, self.width), "embedding")}
+        if self.norm is not None:
+            out[str(self.norm["tensor"])] = TensorSpec((self.width,), "norm")
+        return out
 
     def bind(self, tensors) -> None:
         self.weight = tensors[self.tensor].to(self.rt.device).contiguous()
+        if self.norm is not None:
+            self.norm_weight = tensors[str(self.norm["tensor"])].to(self.rt.device).float().contiguous()
 
     def weight_bytes(self) -> int:
         return 0      # a step reads one row per token, not the table
@@ -36,7 +44,12 @@ class TokenEmbedding(Embedding):
     def forward(self, ctx) -> torch.Tensor:
         x = ctx.ws.buffer("residual", self.width, torch.float32)
         # (a step launched ahead of its tokens names them by the step before: ``ctx.token_feedback``)
-        ops.embed(ctx.tokens[:ctx.rows], self.weight, x, getattr(ctx, "token_feedback", None))
+        if self.norm is None:
+            ops.embed(ctx.tokens[:ctx.rows], self.weight, x, getattr(ctx, "token_feedback", None))
+            return x
+        rows = ctx.ws.buffer("embedded_rows", self.width, torch.float32)
+        ops.embed(ctx.tokens[:ctx.rows], self.weight, rows, getattr(ctx, "token_feedback", None))
+        ops.rmsnorm(rows, self.norm_weight, x, ctx.rows, float(self.norm["eps"]))
         return x
 
 

@@ -21,6 +21,11 @@ padding is zeros).  Further switches:
                            from the request's first token (not together with a window)
     v_mix "source"/"mix"   the first such layer of a model keeps its values of the step's rows ("source"); a later one
                            ("mix") caches v <- (1 - lambda) v + lambda v_source, lambda the tensor ``vmix`` (one number)
+    position layout        a position encoding laid out in "halves" turns element i together with element i + rot/2
+    values "keys"          there is no value projection: a token's values are its keys as projected, before rotation
+    sink "learned"         the sink is a tensor ``sink`` [heads], a number per head
+    gate "head"            the gate is one number per head, sigmoid(W_g h) with W_g [heads, width]
+    window W               the query at position i sees the keys i - W + 1 .. i
   The last taps - 1 projected rows of a request are its state.  Convolution, rotation, norms, scores
 and softmax are 32-bit in both modes; the cache, the queries and the gated output have the mode's activation dtype.
 """
@@ -63,6 +68,13 @@ class GatedAttention(Mixer):
         self.taps = int(p.get("conv") or 0)
         self.whole_norm = p.get("qk_norm") == "whole"
         self.qk_norm, self.gate, self.shared_kv = bool(p.get("qk_norm", False)), bool(p.get("gate", False)), bool(p.get("shared_kv", False))
+        self.head_gate = p.get("gate") == "head"
+        self.values_are_keys = p.get("values") == "keys"
+        if p.get("values") not in (None, "own", "keys"):
+            raise ValueError(f"gated_attention: values are 'own' or 'keys', not {p.get('values')!r}")
+        if self.values_are_keys and (self.dim != self.vdim or self.shared_kv or self.whole_norm or int(p.get("conv") or 0) > 1):
+            raise ValueError("gated_attention: values that are the keys have the keys' size, in a layer with keys of its own, "
+                             "without a convolution or a norm over whole projections")
         self.softcap = float(p.get("softcap") or 0.0)
         self.chunk = int(p.get("chunk") or 0)
         self.v_mix = p.get("v_mix") or None
@@ -72,7 +84,8 @@ class GatedAttention(Mixer):
             raise ValueError("gated_attention: values are mixed by the kernel that norms whole projections, in layers with values of their own")
         if self.softcap < 0 or self.chunk < 0 or (self.chunk and p.get("window")):
             raise ValueError("gated_attention: a soft cap and a chunk are positive; a chunk does not go with a window")
-        self.sink_value: Optional[float] = None if p.get("sink") is None else float(p["sink"])
+        self.learned_sink = p.get("sink") == "learned"
+        self.sink_value: Optional[float] = None if p.get("sink") is None or self.learned_sink else float(p["sink"])
         self.window: Optional[int] = p.get("window")
         if self.heads % self.kv_heads:
             raise ValueError(f"gated_attention: {self.heads} heads are no multiple of {self.kv_heads} kv heads")
@@ -90,17 +103,18 @@ class GatedAttention(Mixer):
         self.rot = 0
         if pos is not None:
             self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
-            if getattr(self.position, "layout", None) != "pairs":
-                raise ValueError(f"gated_attention rotates neighbouring pairs; position encoding '{pos.kind}' is laid out otherwise")
+            if getattr(self.position, "layout", None) not in ("pairs", "halves"):
+                raise ValueError(f"gated_attention rotates neighbouring pairs or halves; position encoding '{pos.kind}' is laid out otherwise")
             self.rot = int(self.position.rotary_dim)
+        self.halves = getattr(self.position, "layout", None) == "halves"
         if self.whole_norm and self.rot:
             raise ValueError("gated_attention: the norm over whole projections comes without rotation")
         if self.rot > self.dim:
             raise ValueError(f"gated_attention: {self.rot} rotated elements in heads of {self.dim}")
         self.q_ch = self.heads * self.dim
-        self.kv_ch = 0 if self.shared_kv else self.kv_heads * (self.dim + self.vdim)
+        self.kv_ch = 0 if self.shared_kv else self.kv_heads * (self.dim + (0 if self.values_are_keys else self.vdim))
         self.conv_ch = self.q_ch + self.kv_ch
-        self.g_ch = self.heads * self.vdim if self.gate else 0
+        self.g_ch = (self.heads if self.head_gate else self.heads * self.vdim) if self.gate else 0
         self.proj: Optional[Linear] = None
         self.o: Optional[Linear] = None
         self.conv_w = self.sink = self.cos = self.sin = None
@@ -110,7 +124,10 @@ class GatedAttention(Mixer):
         out = {"q": TensorSpec((self.q_ch, self.width))}
         if not self.shared_kv:
             out["k"] = TensorSpec((self.kv_heads * self.dim, self.width))
-            out["v"] = TensorSpec((self.kv_heads * self.vdim, self.width))
+            if not self.values_are_keys:
+                out["v"] = TensorSpec((self.kv_heads * self.vdim, self.width))
+        if self.learned_sink:
+            out["sink"] = TensorSpec((self.heads,), "bias")
         if self.taps >= 1:
             out["q.conv"] = TensorSpec((self.q_ch, self.taps), "conv")
             if not self.shared_kv:
@@ -138,7 +155,7 @@ class GatedAttention(Mixer):
             self.k_norm_w = self.q_norm_w if self.shared_kv else tensors["k.norm"].to(dev).float().contiguous()
         if self.v_mix == "mix":
             self.mix_w = tensors["vmix"].to(dev).float().reshape(1).contiguous()
-        names = ["q"] + ([] if self.shared_kv else ["k", "v"]) + (["g"] if self.gate else [])
+        names = ["q"] + ([] if self.shared_kv else (["k"] if self.values_are_keys else ["k", "v"])) + (["g"] if self.gate else [])
         stack = [tensors[n] for n in names]
         if len({t.dtype for t in stack}) != 1:
             raise ValueError("the projections of one mixer must be stored in one dtype to be stacked")
@@ -147,7 +164,9 @@ class GatedAttention(Mixer):
         if self.taps >= 1:
             cn = ["q.conv"] + ([] if self.shared_kv else ["k.conv", "v.conv"])
             self.conv_w = torch.cat([tensors[n].to(dev).float() for n in cn], dim=0).contiguous()      # (widening is exact)
-        if self.sink_value is not None:
+        if self.learned_sink:
+            self.sink = tensors["sink"].to(dev).float().contiguous()
+        elif self.sink_value is not None:
             self.sink = torch.full((self.heads,), self.sink_value, dtype=torch.float32, device=dev)
 
     def weight_bytes(self) -> int:
@@ -198,7 +217,8 @@ class GatedAttention(Mixer):
         else:
             ops.pair_rope_unit(src, ctx.positions, ctx.row_seq, ctx.block_tables[call.group], self.cos, self.sin, q, call.k_cache,
                                call.v_cache, rows, self.heads, self.kv_heads, self.dim, self.vdim, hs, self.rot, ws.page_size,
-                               self.qk_norm, self.eps, not self.shared_kv, call.writes_cache)
+                               self.qk_norm, self.eps, not self.shared_kv, call.writes_cache, halves=self.halves,
+                               values_are_keys=self.values_are_keys)
         av = ws.buffer("gattn_av", self.heads * hs, rt.act_dtype)
         attend = attend_bf16 if rt.bf16 else attend_f32
         attend(ctx, call, q, av, self.heads, self.kv_heads, hs, int(self.window or 0), self.scale, sink=self.sink,
@@ -206,7 +226,7 @@ class GatedAttention(Mixer):
         if self.gate or hs != self.vdim:
             act = ws.buffer("gattn_gated", self.heads * self.vdim, rt.act_dtype)
             if self.gate:
-                ops.gate_mul(av, hs, proj[:, self.conv_ch:], act, rows, self.heads, self.vdim)
+                ops.gate_mul(av, hs, proj[:, self.conv_ch:], act, rows, self.heads, self.vdim, per_head=self.head_gate)
             else:
                 act.view(-1, self.heads, self.vdim)[:rows].copy_(av.view(-1, self.heads, hs)[:rows, :, :self.vdim])
         else:

@@ -1,15 +1,18 @@
 """A feed-forward of routed experts: every row goes through the ``top`` experts its router scores pick, and their
 outputs are added with the scores as weights.
 
-    s       = softmax(W_router h)                              over all experts, 32-bit
-    allowed = the experts of the `keep` best of `groups` equal groups of neighbours (a group's score: its best expert's)
-    chosen  = the `top` allowed experts with the largest s; weights = their s, as they are
+    s       = softmax(W_router h)                              over all experts, 32-bit (``score`` "sigmoid": the sigmoid of each logit)
+    c       = s, or s + correction                             a learned number per expert that enters the choice only
+    allowed = the experts of the `keep` best of `groups` equal groups of neighbours (a group's score: its best c, or
+              with ``group_best`` n the sum of its n best)
+    chosen  = the `top` allowed experts with the largest c; weights = their s, as they are
     expert  : g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), W_down (g sigmoid(alpha g) (u + 1))
               or, with limit None, the plain gated form W_down (g sigmoid(alpha g) u), g = W_gate h, u = W_up h
 
 ``weight_scale`` multiplies the chosen scores.  ``shared`` = {ff}: one more expert of the plain gated form (tensors
 shared.gate, shared.up, shared.down) that every row goes through, its output multiplied by sigmoid(w_sg . h), one number
-a row (tensor shared.sg [1, width]); the gate's product rides under the router's, 32-bit like it.
+a row (tensor shared.sg [1, width]); the gate's product rides under the router's, 32-bit like it.  ``shared`` =
+{ff, "gated": False}: the shared expert's output is added as it is (no tensor shared.sg).
 
 Routing happens on the device and the experts' products run over a plan built there, so a step never waits for the
 host and a captured decode step stays valid.  What a row gets from an expert depends on the row and the expert
@@ -30,9 +33,10 @@ from .linear import Linear
 @register_feed_forward("moe")
 class RoutedExperts(FeedForward):
     """params: width, experts, top, groups (1), keep (groups), ff, limit (None: the plain form), alpha (1.702; 1 makes the
-    plain form SiLU), weight_scale (1), shared (None or {ff}).
+    plain form SiLU), weight_scale (1), shared (None or {ff, gated (True)}), score ("softmax" or "sigmoid"), correction
+    (False; True: a tensor ``correction`` [experts] joins the scores for the choice), group_best (1).
     tensors: router [experts, width]; e<j>.gate, e<j>.up [ff, width]; e<j>.down [width, ff]; with ``shared``:
-    shared.gate, shared.up [ff_s, width], shared.down [width, ff_s], shared.sg [1, width]."""
+    shared.gate, shared.up [ff_s, width], shared.down [width, ff_s], shared.sg [1, width] if gated; correction [experts]."""
 
     graph_safe = True
     launches_through_ops = True
@@ -47,6 +51,15 @@ class RoutedExperts(FeedForward):
         self.alpha = float(p.get("alpha", 1.702))
         self.weight_scale = float(p.get("weight_scale", 1.0))
         self.shared_ff = int(p["shared"]["ff"]) if p.get("shared") else 0
+        self.shared_gated = bool(p["shared"].get("gated", True)) if p.get("shared") else False
+        if p.get("score", "softmax") not in ("softmax", "sigmoid"):
+            raise ValueError(f"moe: scores are 'softmax' or 'sigmoid', not {p.get('score')!r}")
+        self.score = ops.SCORE_SIGMOID if p.get("score") == "sigmoid" else ops.SCORE_SOFTMAX
+        self.has_correction = bool(p.get("correction", False))
+        self.group_best = int(p.get("group_best", 1))
+        if not 1 <= self.group_best <= 4:
+            raise ValueError("moe: a group's score sums one to four of its best")
+        self.correction: Optional[torch.Tensor] = None
         if p.get("limit") is not None and not self.limit > 0:
             raise ValueError("moe: the experts' limit must be positive (None: no limit)")
         if self.experts % self.groups or not 1 <= self.keep <= self.groups:
@@ -69,17 +82,24 @@ class RoutedExperts(FeedForward):
             out["shared.gate"] = TensorSpec((self.shared_ff, self.width))
             out["shared.up"] = TensorSpec((self.shared_ff, self.width))
             out["shared.down"] = TensorSpec((self.width, self.shared_ff))
-            out["shared.sg"] = TensorSpec((1, self.width), "router")
+            if self.shared_gated:
+                out["shared.sg"] = TensorSpec((1, self.width), "router")
+        if self.has_correction:
+            out["correction"] = TensorSpec((self.experts,), "small_bias")
         return out
 
     def bind(self, tensors) -> None:
         dev = self.rt.device
         # the router's sums are 32-bit in either mode; in bfloat16 mode the rows arrive rounded and the weights are stored
         # so, their products are exact in 32 bits and the matrix cores add them up in 32 bits
+        if self.has_correction:
+            self.correction = tensors["correction"].to(dev).float().contiguous()
         if self.shared_ff:
-            if tensors["shared.sg"].dtype != tensors["router"].dtype or tensors["shared.gate"].dtype != tensors["shared.up"].dtype:
+            if tensors["shared.gate"].dtype != tensors["shared.up"].dtype or (
+                    self.shared_gated and tensors["shared.sg"].dtype != tensors["router"].dtype):
                 raise ValueError("the router and the shared expert's gate (and its two branches) must be stored in one dtype to be stacked")
-            self.router = Linear(torch.cat([tensors["router"], tensors["shared.sg"]], dim=0), self.rt)
+            self.router = Linear(torch.cat([tensors["router"], tensors["shared.sg"]], dim=0) if self.shared_gated else tensors["router"],
+                                 self.rt)
             self.shared_gate_up = Linear(torch.cat([tensors["shared.gate"], tensors["shared.up"]], dim=0), self.rt)
             self.shared_down = Linear(tensors["shared.down"], self.rt)
         else:
@@ -120,7 +140,8 @@ class RoutedExperts(FeedForward):
         tiles = ws.buffer("moe_tiles", 4 * (most // 16 + self.experts), torch.int32, rows=1)
         meta = ws.buffer("moe_meta", 4, torch.int32, rows=1)
         ops.moe_route_plan(logits, rows, self.top, self.groups, self.keep, ids, wts, sorted_slots, place, tiles, meta,
-                           weight_scale=self.weight_scale, experts=self.experts)
+                           weight_scale=self.weight_scale, experts=self.experts, score=self.score, correction=self.correction,
+                           group_best=self.group_best)
         if self.mfma:
             x, act_dtype = h, torch.bfloat16
         else:
@@ -135,7 +156,7 @@ class RoutedExperts(FeedForward):
         ops.moe_experts(act, self.down, y, sorted_slots, tiles, meta, slots, self.top, False)
         if norm is not None:
             # the rows' weighted sums are formed by the kernel that norms them and adds them into the stream
-            ops.norm_add(y, norm.weight, target, rows, norm.eps, rounded, combine=(place, wts, self.top))
+            ops.norm_add(y, norm.weight, target, rows, norm.eps, rounded, combine=(place, wts, self.top), scale=norm.scale)
         else:
             ops.moe_combine(y, place, wts, self.top, target, rows, add)
         if self.shared_ff:
@@ -144,7 +165,7 @@ class RoutedExperts(FeedForward):
             gu = ws.buffer("moe_shared_gu", 2 * self.shared_ff, torch.float32)
             self.shared_gate_up.store(ws, h, gu, rows)
             sact = ws.buffer("moe_shared_act", self.shared_ff, rt.act_dtype)
-            ops.glu(gu, sact, rows, ops.ACT_SILU, row_gate=logits[:, self.experts:self.experts + 1])
+            ops.glu(gu, sact, rows, ops.ACT_SILU, row_gate=logits[:, self.experts:self.experts + 1] if self.shared_gated else None)
             self.shared_down.add_into(ws, sact, target, rows)
 
     def forward(self, ctx, h, residual) -> None:

@@ -1,6 +1,6 @@
 """Mixers with a matrix memory per head instead of a cache: S <- decay * S + k v^T, o = S^T q.
 
-Two kinds share the arrangement (one stacked projection of the mixer's input, the recurrence over each request's
+Four kinds share the arrangement (one stacked projection of the mixer's input, the recurrence over each request's
 rows in order from and to its state slot, a per-head RMS norm of the read-out with an output gate, the output
 projection added into the residual stream) and differ in the decay:
 
@@ -9,6 +9,12 @@ projection added into the residual stream) and differ in the decay:
 * ``mlstm``: the matrix memory of the xLSTM, scalar input and forget gates per head in the log domain, capped by
   cap * tanh(. / cap), with a normaliser n and a stabilising maximum m (a new request's m is 0, like the rest of its
   state); the read-out is divided by max(|n.q|, exp(-m)) + 1e-6, the norm weight spans all heads and the gate is a sigmoid.
+* ``wkv``: time mixing in the manner of RWKV: every projection reads its own mix of the token's and the previous token's
+  input (the norm in front of the mixer delivers the mixes side by side), the decay per key channel is
+  exp(-exp(W2 tanh(W1 x) + w0)), and the read-out comes before the update, with the token's own k v^T weighted by a
+  learned bonus: o = (S + diag(u) k v^T)^T r, then S <- diag(decay) S + k v^T; SiLU gate, norm weight over all heads.
+* ``retention``: one constant decay per head, queries and keys rotated by position (halves layout) and the keys scaled by
+  dim^(-1/2) behind the rotation; the read-out norm has no weight and the gate is SiLU.
 
 The state, the gates and everything between the projections and the read-out are 32-bit in both modes; the
 projections' sums arrive as 32-bit values and are not rounded on the way.
@@ -22,7 +28,7 @@ import numpy as np
 import torch
 
 from ..csrc import ops
-from .base import Mixer, StateSpec, TensorSpec, register_mixer
+from .base import Mixer, POSITION_ENCODINGS, StateSpec, TensorSpec, lookup, register_mixer
 from .linear import Linear
 
 
@@ -122,7 +128,7 @@ class _MatrixMemoryMixer(Mixer):
         self.proj.store(ctx.ws, h, y, ctx.rows)
         return y
 
-    def _recur(self, ctx, call, y, gate, gate_off, gate2_off, bias, bias2, param, raw) -> None:
+    def _recur(self, ctx, call, y, gate, gate_off, gate2_off, bias, bias2, param, raw, kscale: float = 1.0) -> None:
         plan = _scan_plan(ctx)
         seq_rows, nseq, scan = ctx.seq_rows, ctx.nseq, None
         if plan is not None:
@@ -134,13 +140,16 @@ class _MatrixMemoryMixer(Mixer):
             scan = (chunks, nchunks, spans, nspans, local, start)
         ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], gate, gate_off, gate2_off,
                               bias, bias2, param, self.qscale, call.state, raw, seq_rows, ctx.slots, ctx.positions, nseq,
-                              self.heads, self.dim, self.vdim, scan=scan)
+                              self.heads, self.dim, self.vdim, scan=scan, kscale=kscale)
 
-    def _finish(self, ctx, y, raw, residual) -> None:
+    def _finish(self, ctx, y, raw, target, add: bool = True) -> None:
         act = ctx.ws.buffer("recur_gated", self.heads * self.vdim, self.rt.act_dtype)
         ops.head_norm_gate(raw, self.norm_weight, self.per_head_norm_weight, y, self.offsets["g"], self.gate_kind, act,
                            ctx.positions, ctx.rows, self.heads, self.vdim, self.eps)
-        self.o.add_into(ctx.ws, act, residual, ctx.rows)
+        if add:
+            self.o.add_into(ctx.ws, act, target, ctx.rows)
+        else:
+            self.o.store(ctx.ws, act, target, ctx.rows)
 
 
 @register_mixer("gla")
@@ -231,3 +240,147 @@ class MatrixLSTM(_MatrixMemoryMixer):
         raw = ctx.ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
         self._recur(ctx, call, y, y, self.offsets["i"], self.offsets["f"], self.i_bias, self.f_bias, self.cap, raw)
         self._finish(ctx, y, raw, residual)
+
+
+@register_mixer("wkv")
+class TimeMixWKV(_MatrixMemoryMixer):
+    """params: width, heads, dim (key and value channels a head), eps, rank (the inner size of the decay's projection),
+    inputs (the names of the mixes the norm in front delivers side by side, in its order; this mixer reads "r", "k", "v",
+    "g" and "w" among them).
+    tensors: r, k, v, g [heads*dim, width]; w1 [rank, width]; w2 [heads*dim, rank]; w0 [heads*dim]; u [heads, dim];
+    norm [heads*dim]; o [width, heads*dim].  The mixer's input is [rows, len(inputs) * width]."""
+
+    mode = ops.RECUR_BONUS_DECAY
+    gate_kind = ops.GATE_SILU
+    per_head_norm_weight = True
+    READS = ("r", "k", "v", "g", "w")
+
+    def __init__(self, params, runtime):
+        params = dict(params, vdim=int(params["dim"]))
+        super().__init__(params, runtime)
+        self.qscale = 1.0                     # (the receptance enters the read-out as it is)
+        self.rank = int(params["rank"])
+        self.inputs = [str(n) for n in params.get("inputs", self.READS)]
+        missing = [n for n in self.READS if n not in self.inputs]
+        if missing or self.rank < 1:
+            raise ValueError(f"wkv: the norm in front must deliver the mixes {missing}; the decay's inner size must be positive")
+        self.lin: Dict[str, Linear] = {}
+        self.w2: Optional[Linear] = None
+        self.w0 = self.bonus = None
+
+    def _stack_sizes(self):
+        hd = self.heads * self.dim
+        return [("r", hd), ("k", hd), ("v", hd), ("g", hd), ("w1", self.rank)]
+
+    def tensors(self):
+        out = super().tensors()
+        hd = self.heads * self.dim
+        out["w2"] = TensorSpec((hd, self.rank))
+        out["w0"] = TensorSpec((hd,), "small_bias")
+        out["u"] = TensorSpec((self.heads, self.dim), "small_bias")
+        return out
+
+    def bind(self, tensors) -> None:
+        dev = self.rt.device
+        off = 0
+        for name, n in self._stack_sizes():
+            self.offsets[name] = off
+            off += n
+            self.lin[name] = Linear(tensors[name], self.rt)
+        self.offsets["q"] = self.offsets["r"]
+        self.proj_width = off
+        # (the decay's second product reads 32-bit values behind the tanh and its inner size is tiny: the 32-bit kernels)
+        self.w2 = Linear(tensors["w2"], self.rt, matrix_cores=False)
+        self.w0 = tensors["w0"].to(dev).float().reshape(-1).contiguous()
+        self.bonus = tensors["u"].to(dev).float().reshape(-1).contiguous()
+        self.o = Linear(tensors["o"], self.rt)
+        self.norm_weight = tensors["norm"].to(dev).float().contiguous()
+
+    def weight_bytes(self) -> int:
+        return sum(l.nbytes() for l in self.lin.values()) + self.w2.nbytes() + self.o.nbytes() + 4 * (
+            self.w0.numel() + self.bonus.numel() + self.norm_weight.numel())
+
+    def _run(self, ctx, call, h, target, add: bool) -> None:
+        ws, rows, W = ctx.ws, ctx.rows, self.width
+        if h.shape[1] != len(self.inputs) * W:
+            raise ValueError(f"wkv: the input must hold {len(self.inputs)} mixes of {W} elements side by side")
+        y = ws.buffer("recur_proj", self.proj_width, torch.float32)
+        for name, n in self._stack_sizes():
+            at = self.inputs.index("w" if name == "w1" else name) * W
+            o = self.offsets[name]
+            self.lin[name].store(ws, h[:, at:at + W], y[:, o:o + n], rows)
+        low = y[:, self.offsets["w1"]:self.offsets["w1"] + self.rank]
+        ops.tanh_rows(low, rows)
+        z = ws.buffer("wkv_decay_logits", self.heads * self.dim, torch.float32)
+        self.w2.store(ws, low, z, rows)
+        raw = ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
+        self._recur(ctx, call, y, z, 0, 0, self.w0, self.bonus, 0.0, raw)
+        self._finish(ctx, y, raw, target, add)
+
+    def forward(self, ctx, call, h, residual) -> None:
+        self._run(ctx, call, h, residual, True)
+
+    def forward_out(self, ctx, call, h, out) -> None:
+        self._run(ctx, call, h, out, False)
+
+
+@register_mixer("retention")
+class Retention(_MatrixMemoryMixer):
+    """params: width, heads, dim, vdim, eps, decay (a number per head), position (PartSpec of a position encoding laid out
+    in halves, or None).  tensors: q, k [heads*dim, width]; v, g [heads*vdim, width]; o [width, heads*vdim]."""
+
+    mode = ops.RECUR_FIXED_DECAY
+    gate_kind = ops.GATE_SILU
+    per_head_norm_weight = False
+
+    def __init__(self, params, runtime):
+        super().__init__(params, runtime)
+        self.kscale, self.qscale = float(self.dim) ** -0.5, 1.0      # (the keys carry the scale, behind their rotation)
+        self.decay_values = [float(d) for d in params["decay"]]
+        if len(self.decay_values) != self.heads or any(not 0.0 <= d <= 1.0 for d in self.decay_values):
+            raise ValueError(f"retention: a decay in [0, 1] for each of the {self.heads} heads is needed")
+        pos = params.get("position")
+        self.position = None
+        self.rot = 0
+        if pos is not None:
+            self.position = lookup(POSITION_ENCODINGS, "position encoding", pos.kind).shared(pos.params, runtime)
+            if getattr(self.position, "layout", None) != "halves":
+                raise ValueError(f"retention rotates halves of a head; position encoding '{pos.kind}' is laid out otherwise")
+            self.rot = int(self.position.rotary_dim)
+            if self.rot > self.dim:
+                raise ValueError(f"retention: {self.rot} rotated elements in heads of {self.dim}")
+        self.decay = self.cos = self.sin = None
+
+    def _stack_sizes(self):
+        hd, hv = self.heads * self.dim, self.heads * self.vdim
+        return [("q", hd), ("k", hd), ("v", hv), ("g", hv)]
+
+    def tensors(self):
+        out = super().tensors()
+        del out["norm"]                       # the read-out is divided by its root mean square and nothing else
+        return out
+
+    def bind(self, tensors) -> None:
+        dev = self.rt.device
+        self._bind_common(dict(tensors, norm=torch.ones(self.vdim)))
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=dev)
+        if self.position is not None:
+            self.cos, self.sin = self.position.tables()
+
+    def weight_bytes(self) -> int:
+        return self.proj.nbytes() + self.o.nbytes()
+
+    def _run(self, ctx, call, h, target, add: bool) -> None:
+        y = self._project(ctx, h)
+        if self.rot:
+            ops.rotate_halves_rows(y, (self.offsets["q"], self.offsets["k"]), self.heads, self.dim, self.rot, self.cos, self.sin,
+                                   ctx.positions, ctx.rows)
+        raw = ctx.ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
+        self._recur(ctx, call, y, None, 0, 0, self.decay, None, 0.0, raw, kscale=self.kscale)
+        self._finish(ctx, y, raw, target, add)
+
+    def forward(self, ctx, call, h, residual) -> None:
+        self._run(ctx, call, h, residual, True)
+
+    def forward_out(self, ctx, call, h, out) -> None:
+        self._run(ctx, call, h, out, False)

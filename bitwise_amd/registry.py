@@ -12,11 +12,13 @@ from typing import Any, Callable, Dict, Mapping, Optional
 from .config import kikarax as kikarax_config
 from .config import kuponex as kuponex_config
 from .config import sepedra as sepedra_config
+from .config import vupolix as vupolix_config
 from .config.llama import ConfigError, LlamaConfig
 from .models.kikarax import TINY_KIKARAX, kikarax_spec
 from .models.kuponex import TINY_KUPONEX, kuponex_spec
 from .models.llama import TINY_LLAMA, llama_spec
 from .models.sepedra import TINY_SEPEDRA, sepedra_spec
+from .models.vupolix import TINY_VUPOLIX, vupolix_spec
 from .parts.base import ModelSpec
 
 
@@ -81,3 +83,5 @@ register_architecture(kuponex_config.ARCHITECTURE, kuponex_config.KuponexConfig.
                       kuponex_config.sizes_from_tensors)
 register_architecture(sepedra_config.ARCHITECTURE, sepedra_config.SepedraConfig.from_dict, sepedra_spec, TINY_SEPEDRA)
 register_architecture(kikarax_config.ARCHITECTURE, kikarax_config.KikaraxConfig.from_dict, kikarax_spec, TINY_KIKARAX)
+register_architecture(vupolix_config.ARCHITECTURE, vupolix_config.VupolixConfig.from_dict, vupolix_spec, TINY_VUPOLIX,
+                      vupolix_config.sizes_from_tensors)
