@@ -250,3 +250,26 @@ def forward(cfg, w, tokens, rnd=identity, stream_out: Optional[list] = None) -> 
         if stream_out is not None:
             stream_out.append(x.clone())
     return (rnd(rms_norm(x, w["final.norm"], eps)) @ w["head"].T) * float(cfg["logit_scale"])
+
+
+def generate_greedy(cfg, w, prompt, new_tokens: int) -> List[int]:
+    """The whole sequence recomputed for every new token; the largest logit wins, the lower index among equals."""
+    toks, out = list(prompt), []
+    for _ in range(new_tokens):
+        nxt = int(torch.argmax(forward(cfg, w, toks)[-1]))
+        toks.append(nxt)
+        out.append(nxt)
+    return out
+
+
+def logits_error(got, want, quantile: float = 1.0) -> float:
+    """Per row: the root mean square of the difference (its mean taken off) over that of the wanted row (its mean taken
+    off); the given quantile over the rows."""
+    g, r = torch.as_tensor(got, dtype=F), torch.as_tensor(want, dtype=F)
+    if not torch.isfinite(g).all():
+        return math.inf
+    d = g - r
+    d = d - d.mean(-1, keepdim=True)
+    c = r - r.mean(-1, keepdim=True)
+    err = torch.sqrt((d * d).mean(-1)) / torch.sqrt((c * c).mean(-1)).clamp_min(1e-30)
+    return float(torch.quantile(err, quantile))

@@ -1,0 +1,581 @@
+"""Vupolix on the GPU against the plain float64 implementation (plain_vupolix): every mechanism alone (kernels and
+one-layer models), whole prompts against token-by-token decoding and against portions down to two tokens, batches of
+unequal requests against each alone with pages and slots that are used again, a key made to stand out far back, at page
+borders and just inside and outside the window (in prompts and in decoding), the sink, memories whose decay is pushed
+to 1, the first tokens, long decoding, and greedy generation through the engine."""
+
+import json
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import bitwise_amd as bw
+import plain_vupolix as pv
+
+pytestmark = pytest.mark.gpu
+
+# float32: 32-bit sums against float64 ones, a few 1e-6 of a row; every row is held.
+# bfloat16: activations rounded where the products take them, carried through the layers and the loop's passes.  A row
+# whose router scores nearly tie picks another expert than the plain model and moves by its own size, and through cache and
+# state the rows behind it move with it.  So in that mode the median over the rows and their 70th percentile are held, and
+# every row only where no router is (the tests of one key that stands out).
+TOL = {"float32": 1e-4, "bfloat16": 0.08}
+WORST_QUANTILE = {"float32": 1.0, "bfloat16": 0.7}
+TYPICAL = {"float32": 2e-5, "bfloat16": 3e-2}
+SIGMA = 0.15
+
+
+def wkv(heads, dim, rank, mlp=None):
+    return {"type": "wkv", "mixer": {"heads": heads, "dim": dim, "rank": rank}, "mlp": mlp}
+
+
+def rot(base, dims, scaling=None):
+    out = {"base": base, "dims": dims}
+    if scaling is not None:
+        out["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return out
+
+
+def par(left, right, mlp=None):
+    """left = (heads, kv_heads, dim, scale, window, rot); right = (heads, dim, vdim, decays, rot)."""
+    lh, lg, ld, ls, lw, lr = left
+    rh, rd, rv, dec, rr = right
+    return {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": lh, "kv_heads": lg, "dim": ld, "vdim": ld, "scale": ls, "mask": {"size": lw}, "rot": lr},
+                      "right": {"heads": rh, "dim": rd, "vdim": rv, "decay": list(dec), "rot": rr}}}
+
+
+def moe(experts, top, ff, groups=None, shared=None):
+    out = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if groups is not None:
+        out["router"]["groups"] = {"count": groups[0], "keep": groups[1]}
+    if shared is not None:
+        out["shared"] = {"ff": shared}
+    return out
+
+
+def config(width, vocab, eps, mult, logit_scale, loop, layers, max_positions=1024):
+    out = {"architecture": "Vupolix", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
+           "logit_scale": logit_scale, "layers": layers, "max_positions": max_positions}
+    if loop is not None:
+        out["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return out
+
+
+YARN = (4.0, 128, 16.0, 2.0)
+CONFIGS = {
+    # one mechanism each
+    "only_wkv": config(48, 61, 1e-5, 1.0, 1.0, None, [wkv(3, 16, 7)]),
+    "only_parallel": config(48, 61, 1e-5, 0.5, 1.0, None, [
+        par((4, 2, 16, 0.4, 21, rot(1000.0, 8, YARN)), (2, 16, 24, (0.9, 0.99), rot(300.0, 16)))]),
+    "only_moe": config(48, 61, 1e-5, 0.7, 2.0, None, [wkv(1, 16, 4, moe(8, 3, 24, (4, 2), 16))]),
+    # a span of layers that runs three times, from the second layer on, and a span that runs once
+    "looped": config(40, 53, 1e-5, 0.3, 1.0, (1, 3, 3), [
+        wkv(2, 8, 3), par((2, 1, 8, 0.5, 9, rot(100.0, 8)), (1, 8, 8, (0.95,), rot(100.0, 4))), wkv(1, 24, 2, moe(4, 2, 8)),
+        wkv(2, 16, 5)]),
+    # sizes that are no multiples of 8 anywhere: every product stays on the 32-bit kernels in bfloat16 mode too, heads are
+    # padded in the cache, groups of one expert
+    "odd": config(44, 53, 1e-5, 0.6, 0.7, (0, 1, 2), [
+        par((3, 1, 20, 0.3, 7, rot(5000.0, 10, (2.5, 50, 9.0, 1.5))), (3, 10, 6, (0.5, 0.9, 1.0), rot(77.0, 6, YARN)), moe(5, 2, 20, (5, 3), 12)),
+        wkv(2, 22, 3, moe(6, 4, 12, (2, 2), None)),
+    ]),
+    # everything together, sizes all different from layer to layer: values wider and narrower than keys, one key head
+    # and as many as query heads, head sizes that the cache pads, windows that are no multiple of a page, wholly and
+    # partly rotated heads, one expert a row and all of them, with and without groups and shared expert, a layer without
+    # feed-forward, the loop in the middle
+    "mixed": config(64, 131, 1e-6, 0.3, 0.5, (1, 4, 2), [
+        wkv(4, 16, 6, moe(6, 1, 40, None, 24)),
+        par((6, 2, 12, 0.5, 37, rot(10000.0, 12, YARN)), (2, 24, 40, (0.97, 0.999), rot(1e6, 24)), moe(9, 3, 16, (3, 2), 8)),
+        wkv(2, 40, 9, None),
+        par((3, 3, 24, 0.3, 50, rot(500.0, 8)), (4, 8, 16, (0.8, 0.9, 0.95, 0.99), rot(50.0, 8, (8.0, 64, 4.0, 1.0))), moe(5, 5, 16)),
+        par((8, 1, 8, 0.7, 16, rot(1000.0, 4)), (1, 32, 8, (0.99,), rot(1000.0, 16)), None),
+    ]),
+    # heads of the sizes real models have, more experts than a wave has lanes, inner sizes beyond one step of the products
+    "wide": config(136, 77, 1e-5, 0.25, 0.5, (0, 2, 2), [
+        wkv(2, 128, 24, moe(72, 6, 48, (8, 3), 64)),
+        par((4, 2, 128, 0.09, 112, rot(50000.0, 64, (4.0, 256, 32.0, 1.0))), (2, 64, 128, (0.98, 0.995), rot(1e6, 64)), moe(3, 2, 136, None, 8)),
+        wkv(4, 64, 16, None),
+    ]),
+}
+SEEDS = {name: 71 + i for i, name in enumerate(CONFIGS)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory, gpu):
+    tmp = tmp_path_factory.mktemp("vupolix")
+    return {name: bw.write_random_model(tmp / name, cfg, SEEDS[name], SIGMA) for name, cfg in CONFIGS.items()}
+
+
+def weights(folder):
+    from safetensors.torch import load_file
+    return pv.to64(load_file(str(Path(folder) / "model.safetensors")))
+
+
+def tokens_for(name, n, seed=0):
+    g = torch.Generator().manual_seed(4000 + seed)
+    return torch.randint(0, CONFIGS[name]["vocab"], (n,), generator=g).tolist()
+
+
+def plain(folder, toks):
+    return pv.forward(json.loads((Path(folder) / "config.json").read_text()), weights(folder), toks).numpy()
+
+
+def close(got, want, dtype):
+    return pv.logits_error(got, want, WORST_QUANTILE[dtype]) < TOL[dtype] and pv.logits_error(got, want, 0.5) < TYPICAL[dtype]
+
+
+def replayer(folder, dtype, max_tokens, **kw):
+    from bitwise_amd.replay import Replayer
+    return Replayer(str(folder), dtype, max_tokens, max_live=4, **kw)
+
+
+def run_cut(rp, rid, toks, cuts):
+    """One request through a replayer in portions of the given sizes (the rest one by one); logits at every position."""
+    out, at = [], 0
+    for n in list(cuts) + [1] * (len(toks) - sum(cuts)):
+        out.append(rp.step([{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}]))
+        at += n
+    rp.step([], [rid])
+    return np.concatenate(out)
+
+
+# ----------------------------------------------------------------------------- the model against the plain one
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_prompts_equal_plain(folders, name, dtype):
+    model = bw.Model.load(folders[name], dtype)
+    for n, seed in ((1, 0), (2, 1), (37, 2), (130, 3)):
+        toks = tokens_for(name, n, seed)
+        assert close(model.logits(toks), plain(folders[name], toks), dtype), (name, n)
+    assert model.weight_bytes > 0 and model.config.width == CONFIGS[name]["width"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "odd", "wide"])
+def test_decoding_and_portions_equal_the_whole_prompt(folders, name, dtype):
+    """Token by token from the first token on, a prompt then single tokens, and portions down to two tokens whose edges
+    fall inside pages and inside windows: every position stays what the plain model says, with graphs and without, and
+    the ways of cutting agree with each other to rounding (float32: 1e-5 of a row)."""
+    toks = tokens_for(name, 83, 5)
+    want = plain(folders[name], toks)
+    cuttings = ([83], [], [51], [2, 2, 3, 16, 17, 2, 30, 5], [15, 1, 1, 33, 2], [64, 2])
+    first = None
+    for graphs in (True, False):
+        rp = replayer(folders[name], dtype, 256, use_graphs=graphs, poison_freed_pages=True)
+        for k, cuts in enumerate(cuttings):
+            got = run_cut(rp, f"r{k}", toks, cuts)
+            assert close(got, want, dtype), (name, graphs, cuts)
+            first = got if first is None else first
+            assert pv.logits_error(got, first, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype]), (name, graphs, cuts)
+        assert rp.manager.all_free()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_portions_in_parallel_passes(folders, dtype):
+    """With the engine's leave to let logits depend on the cut in their last bits, portions of 96 rows and more run
+    their recurrences in three passes over chunks: the same values to rounding, alone and beside short portions."""
+    name = "mixed"
+    toks, other = tokens_for(name, 230, 6), tokens_for(name, 40, 8)
+    want, want_other = plain(folders[name], toks), plain(folders[name], other)
+    rp = replayer(folders[name], dtype, 512, exact_cuts=False)
+    assert close(run_cut(rp, "a", toks, [230]), want, dtype)
+    assert close(run_cut(rp, "b", toks, [100, 3, 127]), want, dtype)
+    lg = rp.step([{"id": "c", "tokens": toks[:200], "want": list(range(200))}, {"id": "d", "tokens": other, "want": list(range(40))}])
+    assert close(lg[:200], want[:200], dtype) and close(lg[200:], want_other, dtype)
+    lg = rp.step([{"id": "c", "tokens": toks[200:], "want": list(range(30))}], ["c", "d"])
+    assert close(lg, want[200:], dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unequal_requests_together_equal_each_alone(folders, dtype):
+    """Four live requests of different lengths, portions beside single tokens, requests that pause, end and are followed
+    by others in the same slots and pages (freed pages are filled with NaN at once): every position as alone, so also
+    what the slots keep between steps (the shifted row, the memories) and what the windows keep in pages."""
+    name = "mixed"
+    lengths = {"a": 70, "b": 9, "c": 33, "d": 1, "e": 48, "f": 21}
+    toks = {r: tokens_for(name, n, 20 + i) for i, (r, n) in enumerate(lengths.items())}
+    want = {r: plain(folders[name], t) for r, t in toks.items()}
+    rp = replayer(folders[name], dtype, 64 * 4, poison_freed_pages=True)
+    plan = [
+        [("a", 17), ("b", 2), ("c", 5), ("d", 1)],
+        [("a", 1), ("b", 1), ("c", 16)],
+        [("a", 30), ("b", 6), ("e", 2)],             # d has ended: e takes its slot; c pauses
+        [("a", 1), ("c", 12), ("e", 31), ("f", 3)],  # b has ended
+        [("a", 21), ("e", 1), ("f", 18)],
+        [("e", 14)],
+    ]
+    at = {r: 0 for r in toks}
+    got = {r: [] for r in toks}
+    slots_used = {}
+    for step in plan:
+        entries, ends = [], []
+        for r, n in step:
+            entries.append({"id": r, "tokens": toks[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == lengths[r]:
+                ends.append(r)
+        lg = rp.step(entries, [])
+        for r in (e["id"] for e in entries):
+            slots_used[r] = rp.live[r].slot
+        row = 0
+        for r, n in step:
+            got[r].append(lg[row:row + n])
+            row += n
+        rp.step([], ends)
+    assert at == lengths and rp.manager.all_free()
+    assert len(set(slots_used.values())) < len(slots_used), "slots were meant to be used again"
+    solo = replayer(folders[name], dtype, 128)
+    for r in toks:
+        assert dtype == "bfloat16" or close(np.concatenate(got[r]), want[r], dtype), r
+        alone = run_cut(solo, r, toks[r], [lengths[r]])
+        assert pv.logits_error(np.concatenate(got[r]), alone, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype]), r
+    assert dtype == "float32" or pv.logits_error(np.concatenate([np.concatenate(got[r]) for r in toks]),
+                                                 np.concatenate([want[r] for r in toks]), 0.5) < TYPICAL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """250 tokens one by one behind a short prompt, across many pages and windows, then most of it as one portion."""
+    name = "wide"
+    toks = tokens_for(name, 280, 7)
+    rp = replayer(folders[name], dtype, 320)
+    got = run_cut(rp, "x", toks, [30])
+    assert close(got, plain(folders[name], toks), dtype)
+    again = run_cut(rp, "y", toks, [250])
+    assert pv.logits_error(again, got, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_engine(folders, dtype):
+    """bw.generate with the engine's scheduler, a small token budget and a small page pool: the tokens of the plain
+    implementation, which recomputes the whole sequence for every token; crowded and alone give the same tokens."""
+    name = "mixed"
+    cfg, w = CONFIGS[name], weights(folders[name])
+    model = bw.Model.load(folders[name], dtype)
+    prompts = [tokens_for(name, n, 40 + n) for n in (1, 6, 19, 40)]
+    sp = bw.SamplingParams(max_new_tokens=10, ignore_eos=True)
+    results = bw.generate(model, prompts, sp, bw.EngineConfig(num_blocks=16, max_batched_tokens=24, max_num_seqs=3, dtype=dtype))
+    for p, r in zip(prompts, results):
+        assert r.finished and len(r.tokens) == 10
+        if dtype == "float32":
+            assert r.tokens == pv.generate_greedy(cfg, w, p, 10)
+    for p, r in zip(prompts, results):
+        solo = bw.generate(model, [p], sp, bw.EngineConfig(num_blocks=16, max_num_seqs=1, dtype=dtype, use_graphs=False))[0]
+        assert solo.tokens == r.tokens
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_randomized_scenarios(gpu, dtype):
+    """The scenario simulator on the architecture's tiny model: every request against its solo run, no page or slot
+    lost; preemption happens on the way and restarts from a cleared slot."""
+    from bitwise_amd.registry import ARCHITECTURES
+    from bitwise_amd.sim import Simulator
+
+    model = bw.Model.random(ARCHITECTURES["Vupolix"].tiny_config, 43, dtype, sigma=0.08)
+    tally = Simulator(model, dtype).run(12, seed=2)
+    print(tally.line(dtype))
+    assert tally.violations() == 0, "\n".join(tally.notes[:10])
+    assert tally.requests_compared > 30 and tally.prefix_hit_tokens == 0
+
+
+# ----------------------------------------------------------------------------- one key made to stand out
+
+def needle_model(tmp, window, sink, tag=""):
+    """One layer of the two side-by-side mixers, no feed-forward, the retention branch silenced (its output projection
+    cleared), token rows that are unit vectors, keys that answer to token A alone and queries to token B alone, in the
+    elements of the heads that are not rotated, with a scale that makes that one score large: what a B sees of an A
+    decides its logits.  The values are the keys, so A's value stands out as well.  Returns (folder, config, A, B, filler)."""
+    from safetensors.torch import load_file, save_file
+    width, vocab = 64, 40
+    a, b, filler = 7, 11, 3
+    layer = par((2, 1, 16, 6.0, window, rot(1000.0, 8)), (1, 8, 8, (0.9,), rot(100.0, 8)))
+    cfg = config(width, vocab, 1e-6, 1.0, 1.0, None, [layer], max_positions=1024)
+    folder = bw.write_random_model(Path(tmp) / f"needle_{window}_{tag}", cfg, 77, 0.02)
+    w = load_file(str(Path(folder) / "model.safetensors"))
+    w["embed"] = torch.eye(vocab, width).to(torch.bfloat16)
+    for n in ("embed.norm", "l0.norm1", "l0.mix.left.out"):
+        w[n] = torch.ones_like(w[n])
+    w["l0.mix.right.o"] = torch.zeros_like(w["l0.mix.right.o"])
+    w["l0.mix.left.sink"] = torch.tensor([sink, 0.0]).to(w["l0.mix.left.sink"].dtype)      # (the first head's; the other's is 0)
+    w["l0.mix.left.g"] = torch.zeros_like(w["l0.mix.left.g"])          # every gate is 1/2
+    g = torch.Generator().manual_seed(5)
+    direction = torch.cat([torch.zeros(8), torch.randn(8, generator=g)])          # the rotated elements stay out of it
+    k = torch.randn(16, width, generator=g)
+    k = 0.01 * (k - torch.outer(direction, direction @ k) / (direction @ direction))     # the other tokens' keys: across the direction
+    k[:, a] = 0.5 * direction
+    q = 0.01 * torch.randn(32, width, generator=g)
+    q[:, b] = 0.5 * torch.cat([direction, direction])
+    w["l0.mix.left.k"], w["l0.mix.left.q"] = k.to(torch.bfloat16), q.to(torch.bfloat16)
+    w["l0.mix.left.o"] = (0.3 * torch.randn(width, 32, generator=g)).to(torch.bfloat16)
+    save_file(w, str(Path(folder) / "model.safetensors"))
+    return folder, cfg, a, b, filler
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [37, 48, 300])
+def test_a_key_that_stands_out(tmp_path_factory, gpu, dtype, window):
+    """One key answers a later query with a large score: far back, at page borders (pages of 16), as the first token, and
+    just inside and just outside the query's window, in a prompt and in decoding.  The test first makes sure, with the
+    plain model, that seeing the key or not moves the logits by far more than the tolerance."""
+    folder, cfg, a, b, filler = needle_model(tmp_path_factory.mktemp("needle"), window, 0.0)
+    w = weights(folder)
+    n = 300
+    W = window
+    # (key position, query position): far back, around page borders, the first token, around the window's edge
+    cases = [(0, n - 1), (0, W - 1), (0, W), (1, W), (1, W + 1), (15, 15 + W - 1), (16, 16 + W - 1), (16, 16 + W), (17, 17 + W),
+             (200 - W, 199), (200 - W, 200), (250, 250 + W - 1), (250, 250 + W), (239, 240), (240, 241), (3, 290)]
+    cases = [(k, q) for k, q in cases if 0 <= k < q < n]
+    seen = unseen = 0
+    rp = replayer(folder, dtype, 320)
+    for i, (kpos, qpos) in enumerate(cases):
+        toks = [filler] * n
+        toks[kpos], toks[qpos] = a, b
+        want = pv.forward(cfg, w, toks).numpy()
+        base = [filler] * n
+        base[qpos] = b
+        without = pv.forward(cfg, w, base).numpy()
+        sees = qpos - kpos < W
+        moved = pv.logits_error(want[qpos:qpos + 1], without[qpos:qpos + 1])
+        assert (moved > 0.2) == sees, (kpos, qpos, moved)
+        seen, unseen = seen + sees, unseen + (not sees)
+        # as a prompt, and with the query (and what lies behind the key) decoded token by token
+        for cuts in ([n], [kpos + 1], [max(qpos - 3, 1), 2]):
+            got = run_cut(rp, f"n{i}", toks, cuts)
+            assert pv.logits_error(got, want, 1.0) < TOL[dtype], (kpos, qpos, cuts)
+    assert seen >= 5 and (unseen >= 5 or window >= n)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_sink_takes_its_share(tmp_path_factory, gpu, dtype):
+    """A large sink leaves a head's keys next to nothing, a very negative one is as good as absent, and a sink of zero counts
+    as one more key of score zero.  The norm behind the mixer hides a factor that all heads share, so the first head's sink
+    is moved and the other's stays: three different models, according to the plain implementation, and the engine follows each."""
+    tmp = tmp_path_factory.mktemp("sink")
+    outs = []
+    for sink in (9.0, 0.0, -30.0):
+        folder, cfg, a, b, filler = needle_model(tmp, 20, sink, tag=f"s{sink}")
+        toks = [filler] * 60
+        toks[30], toks[40], toks[5], toks[59] = a, b, a, b
+        want = pv.forward(cfg, weights(folder), toks).numpy()
+        outs.append(want)
+        rp = replayer(folder, dtype, 128)
+        for cuts in ([60], [35], [2, 2, 37]):
+            assert pv.logits_error(run_cut(rp, "s", toks, cuts), want, 1.0) < TOL[dtype], (sink, cuts)
+    # (judged where the scores are small, in front of the first key that stands out: beside that key no sink of this size counts)
+    assert pv.logits_error(outs[0][:5], outs[1][:5], 0.0) > 0.05 and pv.logits_error(outs[1][:5], outs[2][:5], 0.0) > 0.05
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", ["wkv", "retention"])
+def test_memories_that_do_not_fade(tmp_path_factory, gpu, dtype, kind):
+    """Decays pushed to 1: the first token still moves the logits 250 tokens later (the plain model says so), through
+    prompts, portions and decoding; with the usual decays it would be long gone."""
+    from safetensors.torch import load_file, save_file
+    tmp = tmp_path_factory.mktemp("memory")
+    if kind == "wkv":
+        cfg = config(48, 61, 1e-5, 1.0, 1.0, None, [wkv(2, 16, 4)])
+    else:
+        cfg = config(48, 61, 1e-5, 1.0, 1.0, None, [par((1, 1, 8, 0.3, 4, rot(100.0, 8)), (2, 16, 8, (1.0, 0.9999), rot(1e6, 16)))])
+    folder = bw.write_random_model(tmp / kind, cfg, 5, 0.3)
+    w = load_file(str(Path(folder) / "model.safetensors"))
+    if kind == "wkv":
+        w["l0.mix.w0"] = torch.full_like(w["l0.mix.w0"], -14.0)        # exp(-exp(-14)) is 1 - 8e-7
+        w["l0.mix.w2"] = torch.zeros_like(w["l0.mix.w2"])
+    else:
+        w["l0.mix.left.o"] = torch.zeros_like(w["l0.mix.left.o"])
+    save_file(w, str(Path(folder) / "model.safetensors"))
+    w64 = pv.to64(w)
+    n = 260
+    toks = tokens_for("only_wkv", n, 3)
+    other = [(toks[0] + 1) % 61] + toks[1:]
+    want, want_other = pv.forward(cfg, w64, toks).numpy(), pv.forward(cfg, w64, other).numpy()
+    # (one token among 260 that are all remembered alike: some 1/260 of a row, thirty times the 32-bit tolerance)
+    assert pv.logits_error(want[-5:], want_other[-5:], 0.0) > 3e-3, "the first token was meant to matter at the end"
+    rp = replayer(folder, dtype, 320)
+    for cuts in ([n], [1], [200, 2, 50], [17, 100]):
+        assert pv.logits_error(run_cut(rp, "m", toks, cuts), want, 1.0) < TOL[dtype], cuts
+    rp = replayer(folder, dtype, 320, exact_cuts=False)
+    assert pv.logits_error(run_cut(rp, "m", toks, [n]), want, 1.0) < TOL[dtype]
+
+
+# ----------------------------------------------------------------------------- kernels alone
+
+def _dev(gpu):
+    return lambda x: torch.tensor(x, dtype=torch.int32, device=gpu)
+
+
+def test_shift_with_several_mixes_through_portions_and_slots(gpu):
+    """Norm and token shift with five mixing vectors, portions, single tokens and a slot that changes hands."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(1)
+    for width in (24, 37):
+        nmix, eps = 5, 1e-5
+        wn, mix = torch.randn(width, generator=g), torch.rand(nmix, width, generator=g)
+        seqs = [torch.randn(40, width, generator=g) for _ in range(3)]
+        want = []
+        for s in seqs:
+            h = pv.rms_norm(s.double(), wn.double(), eps)
+            want.append(torch.cat([pv.shifted(h, mix[m].double()) for m in range(nmix)], 1))
+        state = torch.zeros(2, width, device=gpu)
+        dev = _dev(gpu)
+        at = [0, 0, 0]
+        plan = [[(0, 5), (1, 1)], [(1, 2), (0, 1)], [(0, 34), (1, 1)], [(1, 36), (2, 3)], [(2, 1)], [(2, 36)]]
+        slot_of = {0: 0, 1: 1, 2: 0}
+        for step in plan:
+            x, posn, row_seq, seq_rows, slots = [], [], [], [], []
+            for i, (r, n) in enumerate(step):
+                if at[r] == 0:
+                    state[slot_of[r]].zero_()
+                seq_rows += [len(posn), n]
+                x.append(seqs[r][at[r]:at[r] + n])
+                posn += list(range(at[r], at[r] + n))
+                row_seq += [i] * n
+                slots.append(slot_of[r])
+            out = torch.zeros(len(posn), nmix * width, device=gpu)
+            ops.norm_shift(torch.cat(x).to(gpu), wn.to(gpu), mix.to(gpu), state, dev(posn), dev(row_seq), dev(seq_rows), dev(slots),
+                           out, len(posn), eps)
+            o = 0
+            for r, n in step:
+                assert (out[o:o + n].cpu().double() - want[r][at[r]:at[r] + n]).abs().max() < 1e-5, (width, r, at[r], n)
+                o += n
+                at[r] += n
+        assert at == [40, 40, 40]
+
+
+@pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 16), (3, 20, 12), (1, 64, 128), (2, 128, 64), (1, 40, 8)])
+@pytest.mark.parametrize("mode", ["bonus", "fixed"])
+def test_recurrences_against_plain(gpu, mode, heads, dim, vdim):
+    """The two memories alone: whole sequences, portions that continue from the slot, and the three passes over chunks."""
+    from bitwise_amd.csrc import ops
+    if mode == "bonus":
+        vdim = dim
+    g = torch.Generator().manual_seed(heads * 100 + dim)
+    T = 150
+    hd, hv = heads * dim, heads * vdim
+    proj = torch.randn(T, 2 * hd + hv, generator=g) * 0.5
+    q, k, v = proj[:, :hd].double().view(T, heads, dim), proj[:, hd:2 * hd].double().view(T, heads, dim), proj[:, 2 * hd:].double().view(T, heads, vdim)
+    dev = _dev(gpu)
+    if mode == "bonus":
+        z, w0, u = torch.randn(T, hd, generator=g), torch.randn(hd, generator=g) - 1.0, torch.randn(hd, generator=g)
+        decay = torch.exp(-torch.exp(z.double() + w0.double())).view(T, heads, dim)
+        want = pv.wkv_recurrence(q, k, v, decay, u.double().view(heads, dim))
+        args = (ops.RECUR_BONUS_DECAY, z.to(gpu), w0.to(gpu), u.to(gpu), 1.0)
+    else:
+        dec = [0.5 + 0.5 * i / heads for i in range(heads)]
+        want = pv.retention(q, k * dim ** -0.5, v, dec)
+        args = (ops.RECUR_FIXED_DECAY, None, torch.tensor(dec, device=gpu), None, dim ** -0.5)
+    pd = proj.to(gpu)
+    positions = dev(list(range(T)))
+
+    def run(cuts, scan_from=None):
+        state = torch.zeros(2, heads * dim * vdim + 3, device=gpu)[:, 3:]           # (a column slice, as a shared slot gives it)
+        out = torch.zeros(T, hv, device=gpu)
+        at = 0
+        for n in cuts:
+            rows = slice(at, at + n)
+            p, o = pd[rows].contiguous(), torch.zeros(n, hv, device=gpu)
+            gate = None if args[1] is None else args[1][rows].contiguous()
+            scan = None
+            seq_rows, nseq = dev([0, n]), 1
+            if scan_from is not None and n >= scan_from:
+                chunks = [(c0, min(32, n - c0), 0, int(c0 + 32 >= n)) for c0 in range(0, n, 32)]
+                rec = heads * (dim * vdim + dim + 2)
+                scan = (dev(sum(chunks, ())), len(chunks), dev([0, 0, len(chunks)]), 1,
+                        torch.zeros(len(chunks) * rec, device=gpu), torch.zeros(len(chunks) * rec, device=gpu))
+                seq_rows, nseq = dev([0, 0]), 0
+            ops.linear_recurrence(args[0], p, 0, hd, 2 * hd, gate, 0, 0, args[2], args[3], 0.0, 1.0, state, o, seq_rows, dev([1]),
+                                  positions[rows].contiguous(), nseq, heads, dim, vdim, scan=scan, kscale=args[4])
+            out[rows] = o
+            at += n
+        return out.cpu().double().view(T, heads, vdim)
+
+    scale = want.abs().max()
+    for cuts in ([T], [1] * T, [7, 64, 2, 77]):
+        assert (run(cuts) - want).abs().max() / scale < 2e-5, cuts
+    assert (run([T], scan_from=96) - want).abs().max() / scale < 2e-5
+    assert (run([20, 130], scan_from=96) - want).abs().max() / scale < 2e-5
+
+
+def test_half_rotation_and_its_tables(gpu):
+    """Frequencies with and without the ramp, the factor on cosines and sines, and the rotation of two sections in place."""
+    from bitwise_amd.csrc import ops
+    from bitwise_amd.parts.base import PartSpec
+    from bitwise_amd.parts.rope import HalfRotaryTable
+    from bitwise_amd.runtime import Runtime
+    rt = Runtime("float32", gpu)
+    g = torch.Generator().manual_seed(4)
+    for r in (rot(10000.0, 12, YARN), rot(50.0, 8, (8.0, 64, 4.0, 1.0)), rot(1e6, 16), rot(300.0, 6, (2.0, 4096, 64.0, 0.5))):
+        table = HalfRotaryTable(dict(r, max_positions=200), rt)
+        f, mag = pv.rotary_frequencies(r)
+        assert np.allclose(table.frequencies(), f.numpy(), rtol=1e-12) and abs(table.magnitude() - mag) < 1e-12
+        heads, dim, T = 3, 20, 50
+        x = torch.randn(T, 5 + 2 * heads * dim, generator=g)
+        pos = list(range(100, 100 + T))
+        cos, sin = table.tables()
+        xd = x.to(gpu)
+        ops.rotate_halves_rows(xd, (5, 5 + heads * dim), heads, dim, r["dims"], cos, sin, _dev(gpu)(pos), T)
+        for s in range(2):
+            sec = x[:, 5 + s * heads * dim:5 + (s + 1) * heads * dim].double().view(T, heads, dim)
+            want = pv.rotate_halves(sec, 100, r).reshape(T, -1)
+            assert (xd[:, 5 + s * heads * dim:5 + (s + 1) * heads * dim].cpu().double() - want).abs().max() < 1e-5
+        assert torch.equal(xd[:, :5].cpu(), x[:, :5])
+    ramped, _ = pv.rotary_frequencies(rot(10000.0, 12, YARN))
+    bare, _ = pv.rotary_frequencies(rot(10000.0, 12))
+    assert float(ramped[0]) == float(bare[0]) and abs(float(ramped[-1]) * 4.0 - float(bare[-1])) < 1e-15
+
+
+def test_routing_by_corrected_sigmoid_scores(gpu):
+    """Sigmoid scores, a correction that enters the choice and not the weights, groups judged by their two best: against
+    the plain rule, for few rows (one launch with the plan) and many, with corrections that make choice scores negative
+    (an expert outside the kept groups must not win against them)."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(3)
+    for experts, top, count, keep, rows in ((12, 3, 3, 2, 7), (12, 3, 3, 2, 40), (9, 2, 9, 3, 33), (72, 6, 8, 3, 50), (6, 4, 1, 1, 5),
+                                            (10, 4, 2, 1, 21)):
+        z = torch.randn(rows, experts + 1, generator=g) * 2.0
+        z[:, experts] = 50.0                                    # would win every row if it were read as an expert
+        corr = -1.0 - 2.0 * torch.rand(experts, generator=g)     # choice scores below zero throughout
+        ids = torch.zeros(rows, top, dtype=torch.int32, device=gpu)
+        wts = torch.zeros(rows, top, device=gpu)
+        if rows <= 16:
+            most = rows * top
+            tabs = [torch.zeros(most, dtype=torch.int32, device=gpu) for _ in range(2)]
+            tiles = torch.zeros(4 * ops.moe_max_tiles(most, experts), dtype=torch.int32, device=gpu)
+            ops.moe_route_plan(z.to(gpu), rows, top, count, keep, ids, wts, tabs[0], tabs[1], tiles, torch.zeros(4, dtype=torch.int32, device=gpu),
+                               experts=experts, score=ops.SCORE_SIGMOID, correction=corr.to(gpu), group_best=2)
+        else:
+            ops.moe_route(z.to(gpu), rows, top, count, keep, ids, wts, experts=experts, score=ops.SCORE_SIGMOID, correction=corr.to(gpu),
+                          group_best=2)
+        for r in range(rows):
+            want_ids, want_w = pv.route(z[r, :experts].double(), corr.double(), top, count, keep)
+            assert ids[r].tolist() == want_ids, (experts, r)
+            assert (wts[r].cpu().double() - torch.stack(want_w)).abs().max() < 1e-6
+        assert float((torch.sigmoid(z[:, :experts]) + corr).max()) < 0
+
+
+def test_row_operations_of_the_side_by_side_mixer(gpu):
+    """The mean of normed branches, the weighted add of a normed row, and the gate a head."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(6)
+    rows, width, eps = 9, 44, 1e-5
+    ys = [torch.randn(rows, width + 4, generator=g)[:, :width] * s for s in (1.0, 30.0, 0.01)]
+    ws = [torch.randn(width, generator=g) for _ in ys]
+    for n in (1, 2, 3):
+        out = torch.zeros(rows, width, device=gpu)
+        ops.norm_mean([y.to(gpu)[:, :width] for y in ys[:n]], [w.to(gpu) for w in ws[:n]], out, rows, eps)
+        want = sum(pv.rms_norm(y.double(), w.double(), eps) for y, w in zip(ys[:n], ws[:n])) / n
+        assert (out.cpu().double() - want).abs().max() < 1e-5
+    x = torch.randn(rows, width, generator=g)
+    xd = x.to(gpu)
+    ops.norm_add(ys[1].contiguous().to(gpu), ws[0].to(gpu), xd, rows, eps, scale=0.3)
+    assert (xd.cpu().double() - (x.double() + 0.3 * pv.rms_norm(ys[1].double(), ws[0].double(), eps))).abs().max() < 1e-5
+    heads, vdim, hs = 3, 12, 16
+    av, gl = torch.randn(rows, heads * hs, generator=g), torch.randn(rows, heads + 2, generator=g)
+    out = torch.zeros(rows, heads * vdim, device=gpu)
+    ops.gate_mul(av.to(gpu), hs, gl.to(gpu)[:, 2:], out, rows, heads, vdim, per_head=True)
+    want = av.double().view(rows, heads, hs)[:, :, :vdim] * torch.sigmoid(gl[:, 2:].double())[:, :, None]
+    assert (out.cpu().double().view(rows, heads, vdim) - want).abs().max() < 1e-5
