@@ -3,7 +3,7 @@
 random weights and uniform random token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bf16|fp32] [--batch B] [--layers L]
-                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex] [--sepedra] [--kikarax]
+                    [--prefill-tokens T] [--no-points] [--shape smollm2|llama3_8b] [--trace-only] [--decode-phases] [--portion-align A] [--mixed] [--sweep] [--kuponex] [--sepedra] [--kikarax] [--vupolix]
 
 A step is one decode step of the whole engine (scheduler, graph replay of the model, sampling,
 token hand-back) for a batch of B requests that each hold a 2,048-token context.  ``value`` is
@@ -182,6 +182,50 @@ def kikarax_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int
     return 0
 
 
+def vupolix_shape(width: int, expert_ff: int, experts: int = 32, top: int = 4, vocab: int = 32000) -> dict:
+    """A Vupolix of six layers (time mixing and the two side-by-side mixers in turn) of which the third and fourth run
+    twice: eight layer runs.  Time mixing with heads of 64, attention with heads of 128, a quarter as many key heads, half
+    of each head rotated along a ramp and a window of 1,024 keys, retention with heads of 128 x 256, feed-forwards of
+    ``experts`` experts in four groups of which two are kept and a token uses ``top``, beside a shared expert."""
+    heads = width // 128
+    mlp = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}},
+           "shared": {"ff": expert_ff}}
+    time_mix = {"type": "wkv", "mixer": {"heads": width // 64, "dim": 64, "rank": 64}, "mlp": mlp}
+    rh = max(1, width // 256)
+    both = {"type": "parallel", "mlp": mlp, "mixer": {
+        "left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
+                 "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+        "right": {"heads": rh, "dim": 128, "vdim": 256, "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(rh - 1, 1)) for i in range(rh)],
+                  "rot": {"base": 1000000.0, "dims": 128}}}}
+    return {"architecture": "Vupolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.3, "logit_scale": 0.25,
+            "loop": {"start": 2, "stop": 4, "times": 2}, "layers": [time_mix, both] * 3, "max_positions": 16384, "eos_token_id": 2}
+
+
+def vupolix_comparison(bw, torch, steps: int, dtype: str, only: str = "") -> int:
+    """Prefill and decode of Vupolix at two layer sizes beside the Sepedra decoder (recurrent and attention layers over
+    routed experts too) of equal width, depth and experts: one JSON object a line."""
+    from bitwise_amd.measure import PEAK_FLOPS, measure_decode, measure_prefill
+    for name, width, expert_ff in (("2048x(4x2048 of 32)", 2048, 2048), ("4096x(4x3584 of 32)", 4096, 3584)):
+        for arch, cfg in (("Vupolix", vupolix_shape(width, expert_ff)), ("Sepedra", sepedra_shape(width, expert_ff, 2))):
+            if only and only.lower() != arch.lower():
+                continue
+            model = bw.Model.random(cfg, seed=0, dtype=dtype, sigma=0.02, on_device=True)
+            for tokens in (512, 2048):
+                for exact in ((True, False) if arch == "Vupolix" else (True,)):
+                    # (exact_cuts False: the matrix memories run a long portion in three passes over chunks)
+                    m = measure_prefill(bw, torch, model, cfg, dtype, PEAK_FLOPS[dtype], tokens, exact_cuts=exact)
+                    print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "prefill_tokens": tokens, "exact_cuts": exact,
+                                      "ms": m["ms"], "tok_s": m["value"], "frac_of_matrix_peak": m["frac"]}), flush=True)
+            for batch in (1, 8, 64):
+                m = measure_decode(bw, torch, model, cfg, dtype, batch, steps, 4, context=2048)
+                print(json.dumps({"shape": name, "model": arch, "dtype": dtype, "decode_batch": batch, "context": 2048,
+                                  "ms_per_step": m["ms_per_step"], "tok_s": m["tok_s"], "frac_of_8_TBs": m["roofline"]["frac"]}),
+                      flush=True)
+            del model
+            torch.cuda.empty_cache()
+    return 0
+
+
 def sweep(bw, torch, steps: int, dtype: str) -> int:
     """Decode steps over batch and context, prefills over length: in bfloat16 at both shapes, in the 32-bit mode a
     coarser grid at the small one.  One JSON object a line."""
@@ -234,6 +278,9 @@ def main() -> int:
     ap.add_argument("--sepedra", nargs="?", const="both", default="", choices=["both", "sepedra", "llama"],
                     help="print a table instead of the line: prefill and decode of the Sepedra design at two layer sizes beside "
                          "the Llama decoder of equal width and depth with a feed-forward as wide as a token's experts together")
+    ap.add_argument("--vupolix", nargs="?", const="both", default="", choices=["both", "vupolix", "sepedra"],
+                    help="print a table instead of the line: prefill and decode of the Vupolix design at two layer sizes beside "
+                         "the Sepedra decoder of equal width, depth and experts (or one of the two)")
     ap.add_argument("--kikarax", nargs="?", const="both", default="", choices=["both", "kikarax", "llama"],
                     help="print a table instead of the line: prefill and decode of the Kikarax design at two layer sizes beside "
                          "the Llama decoder of equal width, depth and active feed-forward width (or one of the two only)")
@@ -255,6 +302,8 @@ def main() -> int:
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     if args.sweep:
         return sweep(bw, torch, args.steps, dtype)
+    if args.vupolix:
+        return vupolix_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.vupolix == "both" else args.vupolix)
     if args.kikarax:
         return kikarax_comparison(bw, torch, min(args.steps, 32), dtype, "" if args.kikarax == "both" else args.kikarax)
     if args.sepedra:

@@ -187,6 +187,9 @@ int bw_norm_add(const float* y, int ldy, const void* w, int w_is_bf16, float* x,
 // out[r] = (1/n) sum_b norm(y[b][r]) * w[b], n <= 4 (host arrays of device pointers)
 int bw_norm_mean(const float* const* y, const int* ldy, const float* const* w, int n, float* out, int ldo, int rows, int dim,
                  float eps, void* stream);
+// x[r] += scale * norm(that mean; w2, eps2), one launch, for rows of up to 2,048 elements: the bits of bw_norm_mean then bw_norm_add
+int bw_norm_mean_add(const float* const* y, const int* ldy, const float* const* w, int n, float eps, const float* w2, float eps2,
+                     float scale, float* x, int ldx, int rows, int dim, void* stream);
 int bw_softcap(float* x, int ld, int rows, int cols, float cap, void* stream);
 int bw_scale_rows(float* x, int ld, int rows, int cols, float factor, void* stream);      // x *= factor
 // A feed-forward of routed experts (moe.hip).

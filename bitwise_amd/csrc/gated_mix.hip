@@ -547,10 +547,12 @@ struct NormMeanArgs {
   float eps;
 };
 
+template <int N>
 __global__ __launch_bounds__(256) void norm_mean_kernel(NormMeanArgs a) {
-  __shared__ float part[4][4];
+  __shared__ float part[N][4];
   const int row = blockIdx.x, tid = threadIdx.x;
-  for (int b = 0; b < a.n; ++b) {
+#pragma unroll
+  for (int b = 0; b < N; ++b) {
     const float* yr = a.y[b] + (size_t)row * a.ldy[b];
     float acc = 0.0f;
     for (int e = tid; e < a.dim; e += 256) acc = fmaf(yr[e], yr[e], acc);
@@ -558,15 +560,104 @@ __global__ __launch_bounds__(256) void norm_mean_kernel(NormMeanArgs a) {
     if ((tid & 63) == 0) part[b][tid >> 6] = acc;
   }
   __syncthreads();
-  float inv[4];
-  for (int b = 0; b < a.n; ++b)
+  float inv[N];
+#pragma unroll
+  for (int b = 0; b < N; ++b)
     inv[b] = 1.0f / sqrtf((((part[b][0] + part[b][1]) + part[b][2]) + part[b][3]) / (float)a.dim + a.eps);
-  const float share = 1.0f / (float)a.n;
+  const float share = 1.0f / (float)N;
   for (int e = tid; e < a.dim; e += 256) {
     float sum = 0.0f;
-    for (int b = 0; b < a.n; ++b) sum += (a.y[b][(size_t)row * a.ldy[b] + e] * inv[b]) * a.w[b][e];
+#pragma unroll
+    for (int b = 0; b < N; ++b) sum += (a.y[b][(size_t)row * a.ldy[b] + e] * inv[b]) * a.w[b][e];
     a.out[(size_t)row * a.ldo + e] = sum * share;
   }
+}
+
+// x[r] += scale * (z / sqrt(mean(z^2) + eps2) * w2) with z the mean of the normed branches as above: the norm behind the
+// mixer rides in the same launch.  Rows of up to 2,048 elements, whose values stay in registers; the bits of
+// norm_mean_kernel followed by norm_add_kernel.
+template <int N>
+__global__ __launch_bounds__(256) void norm_mean_add_kernel(NormMeanArgs a, const float* __restrict__ w2, float eps2, float scale,
+                                                            float* __restrict__ x, int ldx) {
+  __shared__ float part[N][4];
+  __shared__ float part2[4];
+  constexpr int MAXV = 8;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  float v[N][MAXV], wb[N][MAXV], xo[MAXV], wp[MAXV];
+  // everything the row needs is asked for before anything is used
+#pragma unroll
+  for (int j = 0; j < MAXV; ++j) {
+    const int e = min(tid + 256 * j, a.dim - 1);
+#pragma unroll
+    for (int b = 0; b < N; ++b) {
+      v[b][j] = a.y[b][(size_t)row * a.ldy[b] + e];
+      wb[b][j] = a.w[b][e];
+    }
+    xo[j] = x[(size_t)row * ldx + e];
+    wp[j] = w2[e];
+  }
+#pragma unroll
+  for (int b = 0; b < N; ++b) {
+    // (the order of norm_mean_kernel: a thread's elements ascending in one chain)
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < MAXV; ++j)
+      if (tid + 256 * j < a.dim) acc = fmaf(v[b][j], v[b][j], acc);
+    acc = wave_sum(acc);
+    if ((tid & 63) == 0) part[b][tid >> 6] = acc;
+  }
+  __syncthreads();
+  float inv[N];
+#pragma unroll
+  for (int b = 0; b < N; ++b)
+    inv[b] = 1.0f / sqrtf((((part[b][0] + part[b][1]) + part[b][2]) + part[b][3]) / (float)a.dim + a.eps);
+  const float share = 1.0f / (float)N;
+  float z[MAXV];
+  float acc = 0.0f;
+#pragma unroll
+  for (int j = 0; j < MAXV; ++j) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int b = 0; b < N; ++b) sum += (v[b][j] * inv[b]) * wb[b][j];
+    z[j] = tid + 256 * j < a.dim ? sum * share : 0.0f;
+  }
+#pragma unroll
+  for (int j = 0; j < MAXV; ++j) acc = fmaf(z[j], z[j], acc);
+  acc = wave_sum(acc);
+  if ((tid & 63) == 0) part2[tid >> 6] = acc;
+  __syncthreads();
+  const float inv2 = 1.0f / sqrtf((((part2[0] + part2[1]) + part2[2]) + part2[3]) / (float)a.dim + eps2);
+  float* xr = x + (size_t)row * ldx;
+#pragma unroll
+  for (int j = 0; j < MAXV; ++j) {
+    const int e = tid + 256 * j;
+    if (e < a.dim) {
+      const float normed = (z[j] * inv2) * wp[j];
+      xr[e] = scale == 1.0f ? xo[j] + normed : fmaf(scale, normed, xo[j]);
+    }
+  }
+}
+
+extern "C" int bw_norm_mean_add(const float* const* y, const int* ldy, const float* const* w, int n, float eps, const float* w2,
+                                float eps2, float scale, float* x, int ldx, int rows, int dim, void* stream) {
+  if (rows <= 0) return 0;
+  if (n < 1 || n > 4 || dim <= 0 || dim > 2048 || ldx < dim || w2 == nullptr) return -2;
+  NormMeanArgs a{};
+  for (int b = 0; b < n; ++b) {
+    if (y[b] == nullptr || w[b] == nullptr || ldy[b] < dim) return -2;
+    a.y[b] = y[b];
+    a.w[b] = w[b];
+    a.ldy[b] = ldy[b];
+  }
+  a.n = n;
+  a.dim = dim;
+  a.eps = eps;
+  hipStream_t s = (hipStream_t)stream;
+  if (n == 1) hipLaunchKernelGGL(norm_mean_add_kernel<1>, dim3(rows), dim3(256), 0, s, a, w2, eps2, scale, x, ldx);
+  else if (n == 2) hipLaunchKernelGGL(norm_mean_add_kernel<2>, dim3(rows), dim3(256), 0, s, a, w2, eps2, scale, x, ldx);
+  else if (n == 3) hipLaunchKernelGGL(norm_mean_add_kernel<3>, dim3(rows), dim3(256), 0, s, a, w2, eps2, scale, x, ldx);
+  else hipLaunchKernelGGL(norm_mean_add_kernel<4>, dim3(rows), dim3(256), 0, s, a, w2, eps2, scale, x, ldx);
+  return BW_LAUNCH_CHECK();
 }
 
 extern "C" int bw_norm_mean(const float* const* y, const int* ldy, const float* const* w, int n, float* out, int ldo, int rows,
@@ -585,7 +676,11 @@ extern "C" int bw_norm_mean(const float* const* y, const int* ldy, const float* 
   a.ldo = ldo;
   a.dim = dim;
   a.eps = eps;
-  hipLaunchKernelGGL(norm_mean_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, a);
+  hipStream_t s = (hipStream_t)stream;
+  if (n == 1) hipLaunchKernelGGL(norm_mean_kernel<1>, dim3(rows), dim3(256), 0, s, a);
+  else if (n == 2) hipLaunchKernelGGL(norm_mean_kernel<2>, dim3(rows), dim3(256), 0, s, a);
+  else if (n == 3) hipLaunchKernelGGL(norm_mean_kernel<3>, dim3(rows), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(norm_mean_kernel<4>, dim3(rows), dim3(256), 0, s, a);
   return BW_LAUNCH_CHECK();
 }
 

@@ -82,6 +82,7 @@ _SIGS = {
     "bw_rotate_halves_rows": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "bw_tanh_rows": [c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_norm_mean": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "bw_norm_mean_add": [c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_float, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "bw_linear_recurrence": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
                              c_float, c_float, c_float, c_void_p, c_longlong, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                              c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p],
@@ -932,6 +933,32 @@ def norm_mean(ys: Sequence[torch.Tensor], weights: Sequence[torch.Tensor], out: 
     ld = (c_int * n)(*[y.stride(0) for y in ys])
     _check(_fn("bw_norm_mean")(ctypes.cast(yp, c_void_p), ctypes.cast(ld, c_void_p), ctypes.cast(wp, c_void_p), n, out.data_ptr(),
                                out.stride(0), rows, dim, float(eps), _stream()), "norm_mean")
+
+
+NORM_MEAN_ADD_MAX_WIDTH = 2048     # rows that the fused mean + norm + add keeps in a workgroup's registers
+
+
+def norm_mean_add(ys: Sequence[torch.Tensor], weights: Sequence[torch.Tensor], eps: float, post_weight: torch.Tensor, post_eps: float,
+                  scale: float, x: torch.Tensor, rows: int) -> None:
+    """x[:rows] += scale * (z / sqrt(mean(z^2) + post_eps) * post_weight) with z the mean of ``norm_mean``: one launch, the
+    bits of ``norm_mean`` followed by ``norm_add``.  Rows of up to NORM_MEAN_ADD_MAX_WIDTH elements."""
+    n = len(ys)
+    _need(x, torch.float32, "x")
+    _need(post_weight, torch.float32, "post weight")
+    dim = x.shape[1]
+    if not 1 <= n <= 4 or len(weights) != n or x.shape[0] < rows or dim > NORM_MEAN_ADD_MAX_WIDTH or post_weight.numel() != dim:
+        raise ValueError("norm_mean_add: one to four inputs, a weight vector each, rows of up to 2,048 elements")
+    for y, w in zip(ys, weights):
+        _need_strided(y, torch.float32, "input")
+        _need(w, torch.float32, "weight")
+        if y.shape[1] != dim or y.shape[0] < rows or w.numel() != dim:
+            raise ValueError("norm_mean_add: inputs and weights must have x's width")
+    yp = (c_void_p * n)(*[y.data_ptr() for y in ys])
+    wp = (c_void_p * n)(*[w.data_ptr() for w in weights])
+    ld = (c_int * n)(*[y.stride(0) for y in ys])
+    _check(_fn("bw_norm_mean_add")(ctypes.cast(yp, c_void_p), ctypes.cast(ld, c_void_p), ctypes.cast(wp, c_void_p), n, float(eps),
+                                   post_weight.data_ptr(), float(post_eps), float(scale), x.data_ptr(), x.stride(0), rows, dim,
+                                   _stream()), "norm_mean_add")
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, per_head_weight: bool, g: torch.Tensor, g_off: int, gate: int,

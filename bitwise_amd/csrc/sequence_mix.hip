@@ -100,16 +100,23 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
           dq[e] = hp - hq[e];
           keep[e] = (lq[jj][e] * invl) * wq[jj][e];
         }
-        for (int m = 0; m < nmix; ++m) {
-          const f32x4 mm = m == 0 ? mq[jj] : mv[(size_t)m * nvec + c];
-          f32x4 r;
+        // (the further mixing vectors four at a time: their loads are all asked for before the first is used)
+        for (int m0 = 0; m0 < nmix; m0 += 4) {
+          f32x4 mm[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) r[e] = fmaf(dq[e], mm[e], hq[e]);
-          OT* om = o + (size_t)m * dim;
-          if constexpr (sizeof(OT) == 2) {
-            *reinterpret_cast<u32x2*>(om + 4 * c) = (u32x2){pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
-          } else {
-            *reinterpret_cast<f32x4*>(om + 4 * c) = r;
+          for (int k = 0; k < 4; ++k) mm[k] = m0 + k == 0 ? mq[jj] : mv[(size_t)min(m0 + k, nmix - 1) * nvec + c];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (m0 + k >= nmix) continue;
+            f32x4 r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = fmaf(dq[e], mm[k][e], hq[e]);
+            OT* om = o + (size_t)(m0 + k) * dim;
+            if constexpr (sizeof(OT) == 2) {
+              *reinterpret_cast<u32x2*>(om + 4 * c) = (u32x2){pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+            } else {
+              *reinterpret_cast<f32x4*>(om + 4 * c) = r;
+            }
           }
         }
         if (is_first) reinterpret_cast<f32x4*>(st)[c] = keep;
@@ -136,6 +143,101 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(const float* __restrict
     const float hp = st[i];
     for (int m = 0; m < nmix; ++m) store_act(o + (size_t)m * dim + i, fmaf(hp - h, mix[(size_t)m * dim + i], h));
     st[i] = (xl[i] * invl) * w[i];
+  }
+}
+
+// The same for steps of few rows, a workgroup a row: all of a row's operands (the row, the row before or the slot's, the
+// request's last row, the weight and up to eight mixing vectors) are asked for at once, the rows pass through LDS, and a
+// wave each runs row_sumsq_vec over them from there: the chains, and so the bits, of the kernel above.  Rows of whole
+// 16-byte vectors, up to 4,096 elements.
+#define SHIFT_ROW_MAXV 4
+#define SHIFT_ROW_MAXMIX 8
+template <typename OT>
+__global__ __launch_bounds__(256) void norm_shift_row_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                             const float* __restrict__ mix, float* __restrict__ state,
+                                                             long long state_ld, const int32_t* __restrict__ positions,
+                                                             const int32_t* __restrict__ row_seq,
+                                                             const int32_t* __restrict__ seq_rows,
+                                                             const int32_t* __restrict__ slots, OT* __restrict__ out, int ldo,
+                                                             int rows, int dim, float eps, int nmix) {
+  extern __shared__ float shift_lds[];            // three rows of dim elements, then three numbers
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  if (positions[row] < 0) return;
+  const int seq = row_seq[row];
+  const int first = seq_rows[2 * seq], count = seq_rows[2 * seq + 1];
+  const int slot = slots[seq];
+  if (slot < 0 || count <= 0) return;
+  const float* xr = x + (size_t)row * ldx;
+  float* st = state + (size_t)slot * state_ld;
+  OT* o = out + (size_t)row * ldo;
+  const int nvec = dim >> 2;
+  const bool is_first = row == first;
+  const int last = first + count - 1;
+  const bool need_p = !is_first, need_l = is_first && last != row;
+  const f32x4* xv = reinterpret_cast<const f32x4*>(xr);
+  const f32x4* pv = is_first ? reinterpret_cast<const f32x4*>(st) : reinterpret_cast<const f32x4*>(xr - ldx);
+  const f32x4* lv = reinterpret_cast<const f32x4*>(x + (size_t)last * ldx);
+  const f32x4* wvp = reinterpret_cast<const f32x4*>(w);
+  const f32x4* mv = reinterpret_cast<const f32x4*>(mix);
+  f32x4* sx = reinterpret_cast<f32x4*>(shift_lds);
+  f32x4* sp = sx + nvec;
+  f32x4* sl = sp + nvec;
+  float* invs = reinterpret_cast<float*>(sl + nvec);
+  f32x4 xq[SHIFT_ROW_MAXV], pq[SHIFT_ROW_MAXV], lq[SHIFT_ROW_MAXV], wq[SHIFT_ROW_MAXV], mm[SHIFT_ROW_MAXV][SHIFT_ROW_MAXMIX];
+#pragma unroll
+  for (int j = 0; j < SHIFT_ROW_MAXV; ++j) {
+    const int c = min(tid + 256 * j, nvec - 1);
+    xq[j] = xv[c];
+    pq[j] = pv[c];
+    wq[j] = wvp[c];
+    lq[j] = need_l ? lv[c] : xq[j];
+#pragma unroll
+    for (int m = 0; m < SHIFT_ROW_MAXMIX; ++m) mm[j][m] = mv[(size_t)min(m, nmix - 1) * nvec + c];
+  }
+#pragma unroll
+  for (int j = 0; j < SHIFT_ROW_MAXV; ++j) {
+    const int c = tid + 256 * j;
+    if (c < nvec) {
+      sx[c] = xq[j];
+      if (need_p) sp[c] = pq[j];
+      if (need_l) sl[c] = lq[j];
+    }
+  }
+  __syncthreads();
+  if (wv == 0 || (wv == 1 && need_p) || (wv == 2 && need_l)) {
+    const float ss = row_sumsq_vec(wv == 0 ? sx : (wv == 1 ? sp : sl), nvec, lane);
+    if (lane == 0) invs[wv] = 1.0f / sqrtf(ss / (float)dim + eps);
+  }
+  __syncthreads();
+  const float inv = invs[0];
+  const float invp = need_p ? invs[1] : 1.0f;
+  const float invl = need_l ? invs[2] : inv;
+#pragma unroll
+  for (int j = 0; j < SHIFT_ROW_MAXV; ++j) {
+    const int c = tid + 256 * j;
+    if (c >= nvec) continue;
+    f32x4 hq, dq, keep;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      hq[e] = (xq[j][e] * inv) * wq[j][e];
+      const float hp = is_first ? pq[j][e] : (pq[j][e] * invp) * wq[j][e];
+      dq[e] = hp - hq[e];
+      keep[e] = (lq[j][e] * invl) * wq[j][e];
+    }
+#pragma unroll
+    for (int m = 0; m < SHIFT_ROW_MAXMIX; ++m) {
+      if (m >= nmix) continue;
+      f32x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = fmaf(dq[e], mm[j][m][e], hq[e]);
+      OT* om = o + (size_t)m * dim;
+      if constexpr (sizeof(OT) == 2) {
+        *reinterpret_cast<u32x2*>(om + 4 * c) = (u32x2){pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+      } else {
+        *reinterpret_cast<f32x4*>(om + 4 * c) = r;
+      }
+    }
+    if (is_first) reinterpret_cast<f32x4*>(st)[c] = keep;
   }
 }
 
@@ -573,6 +675,17 @@ extern "C" int bw_norm_shift(const float* x, int ldx, const float* w, const floa
   if (rows <= 0) return 0;
   if (dim <= 0 || nmix < 1 || ldx < dim || (long long)ldo < (long long)nmix * dim || state_ld < dim) return -2;
   hipStream_t s = (hipStream_t)stream;
+  if (rows <= 64 && (dim & 3) == 0 && (ldx & 3) == 0 && (ldo & 3) == 0 && (state_ld & 3) == 0 && dim <= 1024 * SHIFT_ROW_MAXV &&
+      nmix <= SHIFT_ROW_MAXMIX) {
+    const size_t bytes = (size_t)(3 * dim + 4) * sizeof(float);
+    if (out_is_bf16)
+      hipLaunchKernelGGL(norm_shift_row_kernel<bf16_t>, dim3(rows), dim3(256), bytes, s, x, ldx, w, mix, state, state_ld, positions,
+                         row_seq, seq_rows, slots, (bf16_t*)out, ldo, rows, dim, eps, nmix);
+    else
+      hipLaunchKernelGGL(norm_shift_row_kernel<float>, dim3(rows), dim3(256), bytes, s, x, ldx, w, mix, state, state_ld, positions,
+                         row_seq, seq_rows, slots, (float*)out, ldo, rows, dim, eps, nmix);
+    return BW_LAUNCH_CHECK();
+  }
   const dim3 grid((rows + 3) / 4), block(256);
   if (out_is_bf16)
     hipLaunchKernelGGL(norm_shift_kernel<bf16_t>, grid, block, 0, s, x, ldx, w, mix, state, state_ld, positions, row_seq,

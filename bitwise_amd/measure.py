@@ -84,7 +84,36 @@ def kikarax_prefill_flops(cfg: dict, tokens: int) -> float:
     return total + 2 * w * cfg["vocab"]
 
 
+def vupolix_prefill_flops(cfg: dict, tokens: int) -> float:
+    """Multiply-adds times two of one prompt, every layer as often as it runs: every projection (the decay's two, the gates'),
+    the router, the chosen experts and the shared one, the attention's scores and weighted sums over the keys a query sees
+    (its window), and for the memories the update and the read-out of every token (2 x dim x vdim a head each)."""
+    w, total = cfg["width"], 0.0
+    loop = cfg.get("loop") or {"start": 0, "stop": 0, "times": 1}
+    for i, layer in enumerate(cfg["layers"]):
+        m, quadratic = layer["mixer"], 0.0
+        if layer["type"] == "wkv":
+            H, D, R = m["heads"], m["dim"], m.get("rank", 64)
+            per_token = w * (4 * H * D + R) + R * H * D + H * D * w + 2 * H * D * D
+        else:
+            l, r = m["left"], m["right"]
+            H, G, D = l["heads"], l["kv_heads"], l["dim"]
+            per_token = w * (H * D + G * D + H) + H * D * w
+            win = min(l["mask"]["size"], tokens)
+            quadratic = H * 2 * D * (win * (win + 1) / 2 + (tokens - win) * win)
+            per_token += w * r["heads"] * (2 * r["dim"] + 2 * r["vdim"]) + r["heads"] * r["vdim"] * w + 2 * r["heads"] * r["dim"] * r["vdim"]
+        mlp = layer.get("mlp")
+        if mlp:
+            ro = mlp["router"]
+            per_token += w * ro["experts"] + ro["top"] * 3 * w * mlp["expert"]["ff"] + 3 * w * (mlp.get("shared") or {"ff": 0})["ff"]
+        runs = loop["times"] if loop["start"] <= i < loop["stop"] else 1
+        total += runs * 2 * (per_token * tokens + quadratic)
+    return total + 2 * w * cfg["vocab"]
+
+
 def prefill_flops(cfg: dict, tokens: int) -> float:
+    if cfg.get("architecture") == "Vupolix":
+        return vupolix_prefill_flops(cfg, tokens)
     if cfg.get("architecture") == "Kikarax":
         return kikarax_prefill_flops(cfg, tokens)
     if cfg.get("architecture") == "Kuponex":
@@ -285,17 +314,20 @@ def measure_decode(bw, torch, model, cfg: dict, dtype: str, batch: int, steps: i
     assert len(eng.sched.running) == batch
     secs = time_decode(eng, torch, steps, warmup)
     assert len(eng.sched.running) == batch, "a request finished inside the timed steps"
-    kv_token = eng.exec.storage.bytes_per_token()
     # state that a request keeps in a slot is read and written once a step
     storage = eng.exec.storage
+    # keys a decoded token reads, on average: the prompt, what the request decoded while later
+    # prompts were prefilled, the warm-up, and half the timed steps; a cache with a window: no more than the window
+    avg_ctx = context + batch * context / 2048 * (batch - 1) / (2 * batch) + warmup + (steps + 1) / 2
+    kv_read = 0.0
+    for spec, k, v in zip(model.assembled.group_specs, storage.keys, storage.values):
+        per_token = sum(t.shape[0] * (t.shape[2] // storage.page_size) * t.element_size() for t in (k, v))
+        kv_read += per_token * (avg_ctx if spec.window is None else min(avg_ctx, spec.window))
     slot_bytes = sum(t[0].numel() * t.element_size() for t in list(storage.states.values()) + list(storage.block_states.values()))
     del eng, storage
     ms = secs / steps * 1e3
-    # keys a decoded token reads, on average: the prompt, what the request decoded while later
-    # prompts were prefilled, the warm-up, and half the timed steps
-    avg_ctx = context + batch * context / 2048 * (batch - 1) / (2 * batch) + warmup + (steps + 1) / 2
     # (a model of routed experts reads the experts its rows choose: what a step of ``batch`` rows reads on average)
-    step_bytes = model.weight_bytes_for(batch) + batch * avg_ctx * kv_token + 2 * batch * slot_bytes
+    step_bytes = model.weight_bytes_for(batch) + batch * kv_read + 2 * batch * slot_bytes
     achieved = step_bytes / (ms * 1e-3) / 1e9
     return {"tok_s": round(batch * steps / secs, 1), "ms_per_step": round(ms, 4),
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

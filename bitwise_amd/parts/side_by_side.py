@@ -40,6 +40,7 @@ class SideBySide(Mixer):
         self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.branches)
         self.launches_through_ops = all(getattr(b, "launches_through_ops", False) for b in self.branches)
         self.out_weights: List[torch.Tensor] = []
+        self._post_weights: Dict[int, torch.Tensor] = {}      # 32-bit copies of the weights of norms that ride in the last launch
         # where each branch's state lies in the slot: (first element, elements), or None
         self.state_span: List[Optional[Tuple[int, int]]] = []
         at = 0
@@ -112,14 +113,27 @@ class SideBySide(Mixer):
             return calls
         return ctx.memo(("side_by_side_calls", id(self), call.index), make)
 
-    def forward_out(self, ctx, call, h, out) -> None:
-        ws = ctx.ws
+    def _branch_outputs(self, ctx, call, h):
         ys = []
         for i, (b, sub) in enumerate(zip(self.branches, self._branch_calls(ctx, call))):
-            y = ws.buffer(f"side_by_side_{i}", self.width, torch.float32)
+            y = ctx.ws.buffer(f"side_by_side_{i}", self.width, torch.float32)
             b.forward_out(ctx, sub, h, y)
             ys.append(y)
-        ops.norm_mean(ys, self.out_weights, out, ctx.rows, self.eps)
+        return ys
+
+    def forward_out(self, ctx, call, h, out) -> None:
+        ops.norm_mean(self._branch_outputs(ctx, call, h), self.out_weights, out, ctx.rows, self.eps)
+
+    def forward_add_normed(self, ctx, call, h, norm, x) -> bool:
+        """The norm behind the mixer rides in the launch that norms and averages the branches (the same bits)."""
+        from .norm import RMSNorm
+        if type(norm) is not RMSNorm or self.width > ops.NORM_MEAN_ADD_MAX_WIDTH:
+            return False
+        w32 = self._post_weights.get(id(norm))
+        if w32 is None:
+            w32 = self._post_weights[id(norm)] = norm.weight.float().contiguous()       # (widening is exact)
+        ops.norm_mean_add(self._branch_outputs(ctx, call, h), self.out_weights, self.eps, w32, norm.eps, norm.scale, x, ctx.rows)
+        return True
 
     def forward(self, ctx, call, h, residual) -> None:
         y = ctx.ws.buffer("side_by_side_mean", self.width, torch.float32)

@@ -446,6 +446,35 @@ def test_shift_with_several_mixes_through_portions_and_slots(gpu):
         assert at == [40, 40, 40]
 
 
+def test_shift_of_few_rows_and_of_many_leave_the_same_bits(gpu):
+    """Steps of few rows run the shift a workgroup a row, longer ones a wave a row: a request's rows in one step of 200, in
+    steps of up to 64 and one by one come out bit for bit alike, and so does the slot's row."""
+    from bitwise_amd.csrc import ops
+    g = torch.Generator().manual_seed(8)
+    dev = _dev(gpu)
+    for width, nmix in ((256, 5), (2048, 5), (1000, 1), (4096, 8)):
+        T = 200
+        x, wn, mix = torch.randn(T, width, generator=g).to(gpu), torch.randn(width, generator=g).to(gpu), torch.rand(nmix, width, generator=g).to(gpu)
+        outs, states = [], []
+        for cuts in ([T], [64, 3, 60, 1, 40, 32], [1] * T):
+            state = torch.zeros(1, width, device=gpu)
+            out = torch.zeros(T, nmix * width, dtype=torch.bfloat16, device=gpu)
+            at = 0
+            for n in cuts:
+                o = torch.zeros(n, nmix * width, dtype=torch.bfloat16, device=gpu)
+                ops.norm_shift(x[at:at + n].contiguous(), wn, mix, state, dev(list(range(at, at + n))), dev([0] * n), dev([0, n]), dev([0]),
+                               o, n, 1e-6)
+                out[at:at + n] = o
+                at += n
+            outs.append(out)
+            states.append(state.clone())
+        for o, s in zip(outs[1:], states[1:]):
+            assert torch.equal(o.view(torch.int16), outs[0].view(torch.int16)) and torch.equal(s, states[0]), (width, nmix)
+        h = pv.rms_norm(x.cpu().double(), wn.cpu().double(), 1e-6)
+        want = torch.cat([pv.shifted(h, mix[m].cpu().double()) for m in range(nmix)], 1)
+        assert (outs[0].cpu().double() - want).abs().max() < 0.05
+
+
 @pytest.mark.parametrize("heads,dim,vdim", [(2, 16, 16), (3, 20, 12), (1, 64, 128), (2, 128, 64), (1, 40, 8)])
 @pytest.mark.parametrize("mode", ["bonus", "fixed"])
 def test_recurrences_against_plain(gpu, mode, heads, dim, vdim):
@@ -569,6 +598,16 @@ def test_row_operations_of_the_side_by_side_mixer(gpu):
         ops.norm_mean([y.to(gpu)[:, :width] for y in ys[:n]], [w.to(gpu) for w in ws[:n]], out, rows, eps)
         want = sum(pv.rms_norm(y.double(), w.double(), eps) for y, w in zip(ys[:n], ws[:n])) / n
         assert (out.cpu().double() - want).abs().max() < 1e-5
+    # mean, norm and add in one launch: the bits of the two launches
+    for n, width2 in ((2, width), (3, 2048), (2, 1000)):
+        ys2 = [torch.randn(rows, width2, generator=g).to(gpu) for _ in range(n)]
+        ws2 = [torch.randn(width2, generator=g).to(gpu) for _ in range(n + 1)]
+        x0 = torch.randn(rows, width2, generator=g).to(gpu)
+        apart, mean, fused = x0.clone(), torch.zeros(rows, width2, device=gpu), x0.clone()
+        ops.norm_mean(ys2, ws2[:n], mean, rows, eps)
+        ops.norm_add(mean, ws2[n], apart, rows, 1e-6, scale=0.3)
+        ops.norm_mean_add(ys2, ws2[:n], eps, ws2[n], 1e-6, 0.3, fused, rows)
+        assert torch.equal(apart, fused), (n, width2)
     x = torch.randn(rows, width, generator=g)
     xd = x.to(gpu)
     ops.norm_add(ys[1].contiguous().to(gpu), ws[0].to(gpu), xd, rows, eps, scale=0.3)
