@@ -128,7 +128,9 @@ class _MatrixMemoryMixer(Mixer):
         self.proj.store(ctx.ws, h, y, ctx.rows)
         return y
 
-    def _recur(self, ctx, call, y, gate, gate_off, gate2_off, bias, bias2, param, raw, kscale: float = 1.0) -> None:
+    def _recur(self, ctx, call, y, gate, gate_off, gate2_off, bias, bias2, param, raw, kscale: float = 1.0, at=None) -> None:
+        """``at``: where q (or r), k and v lie in a row of ``y``, if not at the stacked projection's own offsets."""
+        at = self.offsets if at is None else at
         plan = _scan_plan(ctx)
         seq_rows, nseq, scan = ctx.seq_rows, ctx.nseq, None
         if plan is not None:
@@ -138,13 +140,13 @@ class _MatrixMemoryMixer(Mixer):
             local = ctx.ws.buffer("recur_scan_local", most * rec, torch.float32, rows=1)
             start = ctx.ws.buffer("recur_scan_start", most * rec, torch.float32, rows=1)
             scan = (chunks, nchunks, spans, nspans, local, start)
-        ops.linear_recurrence(self.mode, y, self.offsets["q"], self.offsets["k"], self.offsets["v"], gate, gate_off, gate2_off,
+        ops.linear_recurrence(self.mode, y, at["r"] if "q" not in at else at["q"], at["k"], at["v"], gate, gate_off, gate2_off,
                               bias, bias2, param, self.qscale, call.state, raw, seq_rows, ctx.slots, ctx.positions, nseq,
                               self.heads, self.dim, self.vdim, scan=scan, kscale=kscale)
 
-    def _finish(self, ctx, y, raw, target, add: bool = True) -> None:
+    def _finish(self, ctx, y, raw, target, add: bool = True, g_off: Optional[int] = None) -> None:
         act = ctx.ws.buffer("recur_gated", self.heads * self.vdim, self.rt.act_dtype)
-        ops.head_norm_gate(raw, self.norm_weight, self.per_head_norm_weight, y, self.offsets["g"], self.gate_kind, act,
+        ops.head_norm_gate(raw, self.norm_weight, self.per_head_norm_weight, y, self.offsets["g"] if g_off is None else g_off, self.gate_kind, act,
                            ctx.positions, ctx.rows, self.heads, self.vdim, self.eps)
         if add:
             self.o.add_into(ctx.ws, act, target, ctx.rows)
@@ -280,13 +282,20 @@ class TimeMixWKV(_MatrixMemoryMixer):
         out["u"] = TensorSpec((self.heads, self.dim), "small_bias")
         return out
 
+    FEW_ROWS = 12          # steps of up to this many rows run the five projections as one product (below)
+
     def bind(self, tensors) -> None:
         dev = self.rt.device
+        names = [name for name, _ in self._stack_sizes()]
+        if len({tensors[n].dtype for n in names}) != 1:
+            raise ValueError("the projections of one mixer must be stored in one dtype to be stacked")
+        # one stacked matrix on the device; every projection is a block of its rows (no second copy)
+        self.stack = Linear(torch.cat([tensors[n].to(dev) for n in names], dim=0), self.rt)
         off = 0
         for name, n in self._stack_sizes():
             self.offsets[name] = off
+            self.lin[name] = Linear(self.stack.weight[off:off + n], self.rt)
             off += n
-            self.lin[name] = Linear(tensors[name], self.rt)
         self.offsets["q"] = self.offsets["r"]
         self.proj_width = off
         # (the decay's second product reads 32-bit values behind the tanh and its inner size is tiny: the 32-bit kernels)
@@ -297,25 +306,38 @@ class TimeMixWKV(_MatrixMemoryMixer):
         self.norm_weight = tensors["norm"].to(dev).float().contiguous()
 
     def weight_bytes(self) -> int:
-        return sum(l.nbytes() for l in self.lin.values()) + self.w2.nbytes() + self.o.nbytes() + 4 * (
+        return self.stack.nbytes() + self.w2.nbytes() + self.o.nbytes() + 4 * (
             self.w0.numel() + self.bonus.numel() + self.norm_weight.numel())
 
     def _run(self, ctx, call, h, target, add: bool) -> None:
         ws, rows, W = ctx.ws, ctx.rows, self.width
         if h.shape[1] != len(self.inputs) * W:
             raise ValueError(f"wkv: the input must hold {len(self.inputs)} mixes of {W} elements side by side")
-        y = ws.buffer("recur_proj", self.proj_width, torch.float32)
-        for name, n in self._stack_sizes():
-            at = self.inputs.index("w" if name == "w1" else name) * W
-            o = self.offsets[name]
-            self.lin[name].store(ws, h[:, at:at + W], y[:, o:o + n], rows)
-        low = y[:, self.offsets["w1"]:self.offsets["w1"] + self.rank]
+        nin, N = len(self.inputs), self.proj_width
+        # (not where the product would first widen its rows into a buffer of the step's size)
+        if rows <= self.FEW_ROWS and h.is_contiguous() and (self.stack.mfma or h.dtype == torch.float32):
+            # Few rows: a launch costs more than its arithmetic, so the stacked matrix meets all the mixes of all the rows in
+            # one product (the shifted rows read as rows * mixes rows of the model's width) and every projection is picked
+            # from the rows of its own mix: row r's projection s lies at column s_mix * N + offset_s of a row of nin * N
+            # columns.  A product's row does not depend on the rows beside it, so these are the bits of a product each.
+            y = ws.buffer("recur_proj_few", N, torch.float32, rows=self.FEW_ROWS * nin)
+            self.stack.store(ws, h.view(-1, W), y, rows * nin)
+            y = y.view(self.FEW_ROWS, nin * N)
+            at = {name: self.inputs.index("w" if name == "w1" else name) * N + self.offsets[name] for name, _ in self._stack_sizes()}
+        else:
+            y = ws.buffer("recur_proj", N, torch.float32)
+            for name, n in self._stack_sizes():
+                src = self.inputs.index("w" if name == "w1" else name) * W
+                o = self.offsets[name]
+                self.lin[name].store(ws, h[:, src:src + W], y[:, o:o + n], rows)
+            at = dict(self.offsets)
+        low = y[:, at["w1"]:at["w1"] + self.rank]
         ops.tanh_rows(low, rows)
         z = ws.buffer("wkv_decay_logits", self.heads * self.dim, torch.float32)
         self.w2.store(ws, low, z, rows)
         raw = ws.buffer("recur_out", self.heads * self.vdim, torch.float32)
-        self._recur(ctx, call, y, z, 0, 0, self.w0, self.bonus, 0.0, raw)
-        self._finish(ctx, y, raw, target, add)
+        self._recur(ctx, call, y, z, 0, 0, self.w0, self.bonus, 0.0, raw, at=at)
+        self._finish(ctx, y, raw, target, add, g_off=at["g"])
 
     def forward(self, ctx, call, h, residual) -> None:
         self._run(ctx, call, h, residual, True)

@@ -247,6 +247,9 @@ def test_long_decoding(folders, dtype):
     assert close(got, plain(folders[name], toks), dtype)
     again = run_cut(rp, "y", toks, [250])
     assert pv.logits_error(again, got, WORST_QUANTILE[dtype]) < (1e-5 if dtype == "float32" else TOL[dtype])
+    # the kernels of prompt portions and those of single tokens (the shift a workgroup a row, the five projections as one
+    # product) leave the same bits
+    assert np.array_equal(again, got)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
