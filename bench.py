@@ -196,8 +196,8 @@ def vupolix_shape(width: int, expert_ff: int, experts: int = 32, top: int = 4, v
         "left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024},
                  "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
         "right": {"heads": rh, "dim": 128, "vdim": 256, "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(rh - 1, 1)) for i in range(rh)],
-                  "rot": {"base": 1000000.0, "dims": 128}}}}
-    return {"architecture": "Vupolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.3, "logit_scale": 0.25,
+                  "rot": {"base": 200000.0, "dims": 128}}}}
+    return {"architecture": "Vupolix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.25, "logit_scale": 0.25,
             "loop": {"start": 2, "stop": 4, "times": 2}, "layers": [time_mix, both] * 3, "max_positions": 16384, "eos_token_id": 2}
 
 
