@@ -983,8 +983,8 @@ def glu(gate_up: torch.Tensor, out: torch.Tensor, rows: int, act: int, limit: fl
     """out = act(gate) * up of the stacked 32-bit product [rows, >= 2*inter] (gate at column 0, up at column inter); out
     float32 or bfloat16 (one rounding).  ACT_CLAMPED_SWISH: g = min(gate, limit), u = clamp(up, -limit, limit),
     out = g sigmoid(alpha g) (u + 1).  ``row_gate`` (a 32-bit column, one number a row): out's row r is multiplied by
-    sigmoid(row_gate[r])."""
-    _need(gate_up, torch.float32, "gate_up")
+    sigmoid(row_gate[r]).  ``gate_up`` may be a column slice of a wider matrix."""
+    _need_strided(gate_up, torch.float32, "gate_up")
     inter = out.shape[1]
     if gate_up.shape[1] < 2 * inter or gate_up.shape[0] < rows or out.shape[0] < rows:
         raise ValueError("glu: gate_up must be [rows, 2*inter] for out [rows, inter]")

@@ -68,7 +68,8 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"moe: {self.top} experts a row out of {self.keep} groups of {self.experts // self.groups}")
         self.router: Optional[Linear] = None
         self.gate_up = self.down = None
-        self.shared_gate_up: Optional[Linear] = None
+        self.shared_gate_up: Optional[Linear] = None       # (None with a shared expert: its two branches ride under the router)
+        self.shared_at = 0                                 # the column of the router's product where they begin
         self.shared_down: Optional[Linear] = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
@@ -98,9 +99,15 @@ class RoutedExperts(FeedForward):
             if tensors["shared.gate"].dtype != tensors["shared.up"].dtype or (
                     self.shared_gated and tensors["shared.sg"].dtype != tensors["router"].dtype):
                 raise ValueError("the router and the shared expert's gate (and its two branches) must be stored in one dtype to be stacked")
-            self.router = Linear(torch.cat([tensors["router"], tensors["shared.sg"]], dim=0) if self.shared_gated else tensors["router"],
-                                 self.rt)
-            self.shared_gate_up = Linear(torch.cat([tensors["shared.gate"], tensors["shared.up"]], dim=0), self.rt)
+            under = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_gated else [])
+            if tensors["shared.gate"].dtype == tensors["router"].dtype:
+                # one product gives the experts' logits, the shared expert's gate and its two branches: all read the same
+                # rows and all leave 32-bit sums (a product's column does not depend on the columns beside it)
+                self.router = Linear(torch.cat(under + [tensors["shared.gate"], tensors["shared.up"]], dim=0), self.rt)
+                self.shared_at = sum(t.shape[0] for t in under)
+            else:
+                self.router = Linear(torch.cat(under, dim=0), self.rt)
+                self.shared_gate_up = Linear(torch.cat([tensors["shared.gate"], tensors["shared.up"]], dim=0), self.rt)
             self.shared_down = Linear(tensors["shared.down"], self.rt)
         else:
             self.router = Linear(tensors["router"], self.rt)
@@ -117,7 +124,9 @@ class RoutedExperts(FeedForward):
         return self.router.nbytes() + self.top * per + self._shared_bytes()
 
     def _shared_bytes(self) -> int:
-        return self.shared_gate_up.nbytes() + self.shared_down.nbytes() if self.shared_ff else 0
+        if not self.shared_ff:
+            return 0
+        return (0 if self.shared_gate_up is None else self.shared_gate_up.nbytes()) + self.shared_down.nbytes()
 
     def weight_bytes_rows(self, rows: int) -> int:
         """Bytes a decode step of ``rows`` rows reads: the router and the experts the rows touch, on average, if every
@@ -162,8 +171,11 @@ class RoutedExperts(FeedForward):
         if self.shared_ff:
             # the shared expert: its activation takes the row's gate with it, so that its down projection adds straight
             # into the target
-            gu = ws.buffer("moe_shared_gu", 2 * self.shared_ff, torch.float32)
-            self.shared_gate_up.store(ws, h, gu, rows)
+            if self.shared_gate_up is None:
+                gu = logits[:, self.shared_at:self.shared_at + 2 * self.shared_ff]
+            else:
+                gu = ws.buffer("moe_shared_gu", 2 * self.shared_ff, torch.float32)
+                self.shared_gate_up.store(ws, h, gu, rows)
             sact = ws.buffer("moe_shared_act", self.shared_ff, rt.act_dtype)
             ops.glu(gu, sact, rows, ops.ACT_SILU, row_gate=logits[:, self.experts:self.experts + 1] if self.shared_gated else None)
             self.shared_down.add_into(ws, sact, target, rows)
