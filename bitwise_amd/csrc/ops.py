@@ -828,7 +828,7 @@ def linear_recurrence(mode: int, proj: torch.Tensor, q_off: int, k_off: int, v_o
     chunk from zero, a walk over a request's chunks that gives each its starting state, each chunk from there), with
     ``local`` and ``start`` float32 of n * heads * (dim*vdim + dim + 2) elements each; ``seq_rows`` then carries no rows
     for those requests (nseq may be 0).  The result differs from the one-pass order by the rounding of the walk's sums."""
-    _need(proj, torch.float32, "proj")
+    _need_strided(proj, torch.float32, "proj")            # (may be a column slice of a wider product)
     if mode != RECUR_FIXED_DECAY:
         _need(gate, torch.float32, "gate")
     _need(bias, torch.float32, "bias")
@@ -891,8 +891,8 @@ def rotate_halves_rows(x: torch.Tensor, offsets: Sequence[int], heads: int, dim:
                        sin: torch.Tensor, positions: torch.Tensor, rows: int) -> None:
     """One or two sections of ``x`` (float32 [rows, >= off + heads*dim], a section at each of ``offsets``) turned in place
     by the rows' positions: of every head's first ``rot`` elements, element i is paired with element i + rot/2; the
-    tables are [positions, rot/2]."""
-    _need(x, torch.float32, "x")
+    tables are [positions, rot/2].  ``x`` may be a column slice of a wider matrix."""
+    _need_strided(x, torch.float32, "x")
     _need(positions, torch.int32, "positions")
     if rot == 0 or rows <= 0:
         return
@@ -966,7 +966,7 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, per_head_weight: bool,
     """out[r, h] = o[r, h] / rms(o[r, h]) * weight * gate(g[r, g_off + h*vdim ..]); weight [heads*vdim] or [vdim]."""
     _need(o, torch.float32, "o")
     _need(weight, torch.float32, "weight")
-    _need(g, torch.float32, "g")
+    _need_strided(g, torch.float32, "g")
     _need(positions, torch.int32, "positions")
     if weight.numel() != (heads * vdim if per_head_weight else vdim) or o.shape[1] != heads * vdim or out.shape[1] != heads * vdim:
         raise ValueError("head_norm_gate: weight, o or out do not fit heads x vdim")

@@ -259,6 +259,13 @@ class Mixer(Part):
         norm and ``forward`` one after the other.  The result must be the same bits."""
         return False
 
+    def input_projection(self):
+        """Optional: the ``Linear`` whose product of the mixer's input (32-bit sums) is all the mixer reads of its input, or
+        None.  A mixer that names one also takes ``adopt_input_projection(weight)`` (the same rows, now a block of a larger
+        matrix: it must keep no copy) and ``forward_out_projected(ctx, call, proj, out)`` (``forward_out`` from the product's
+        columns, a slice of a wider matrix): mixers that stand side by side on one input then share one product."""
+        return None
+
     def forward_add_normed(self, ctx, call, h, norm, x) -> bool:
         """Optional: x += norm(mixer(h)) with the norm behind the mixer riding in the mixer's last kernel.  Return False
         (and do nothing) if this part or this norm cannot; the block then calls ``forward_out`` and the norm one after

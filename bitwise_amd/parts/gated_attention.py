@@ -181,13 +181,26 @@ class GatedAttention(Mixer):
     def state_spec(self) -> Optional[StateSpec]:
         return StateSpec(((self.taps - 1) * self.conv_ch,), "float32") if self.taps > 1 else None
 
-    def _run(self, ctx, call, h, target, add: bool, normed_from=None) -> None:
-        """``normed_from`` = (x, norm) instead of ``h``: the norm rides in the projections' product."""
+    def input_projection(self):
+        # (the plain arrangement only: rotation, cache write and gate read the product's columns by their stride)
+        return self.proj if self.proj is not None and self.taps < 1 and not self.whole_norm else None
+
+    def adopt_input_projection(self, weight) -> None:
+        self.proj = Linear(weight, self.rt)
+
+    def forward_out_projected(self, ctx, call, proj, out) -> None:
+        self._run(ctx, call, None, out, False, projected=proj)
+
+    def _run(self, ctx, call, h, target, add: bool, normed_from=None, projected=None) -> None:
+        """``normed_from`` = (x, norm) instead of ``h``: the norm rides in the projections' product.  ``projected``: the
+        projections' 32-bit sums, already made (columns of a wider product)."""
         rt, ws, rows = self.rt, ctx.ws, ctx.rows
         if self.shared_kv == bool(call.writes_cache):
             raise ValueError("gated_attention: a layer with keys and values of its own writes its cache, one without reads another's")
-        proj = ws.buffer("gattn_proj", self.proj.out_features, torch.float32)
-        if normed_from is not None:
+        proj = projected if projected is not None else ws.buffer("gattn_proj", self.proj.out_features, torch.float32)
+        if projected is not None:
+            pass
+        elif normed_from is not None:
             x, norm = normed_from
             ops.norm_gemm_bf16(x, norm.weight, norm.eps, self.proj.weight, proj, rows, ops.EPI_F32)
         else:

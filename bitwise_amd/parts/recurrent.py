@@ -122,6 +122,12 @@ class _MatrixMemoryMixer(Mixer):
             n += self.heads * self.dim + self.heads
         return StateSpec((n,), "float32")
 
+    def input_projection(self):
+        return self.proj
+
+    def adopt_input_projection(self, weight) -> None:
+        self.proj = Linear(weight, self.rt)
+
     def _project(self, ctx, h) -> torch.Tensor:
         """The stacked projection of the rows as 32-bit sums."""
         y = ctx.ws.buffer("recur_proj", self.proj_width, torch.float32)
@@ -309,6 +315,9 @@ class TimeMixWKV(_MatrixMemoryMixer):
         return self.stack.nbytes() + self.w2.nbytes() + self.o.nbytes() + 4 * (
             self.w0.numel() + self.bonus.numel() + self.norm_weight.numel())
 
+    def input_projection(self):
+        return None                           # (every projection reads a mix of its own)
+
     def _run(self, ctx, call, h, target, add: bool) -> None:
         ws, rows, W = ctx.ws, ctx.rows, self.width
         if h.shape[1] != len(self.inputs) * W:
@@ -392,8 +401,11 @@ class Retention(_MatrixMemoryMixer):
     def weight_bytes(self) -> int:
         return self.proj.nbytes() + self.o.nbytes()
 
-    def _run(self, ctx, call, h, target, add: bool) -> None:
-        y = self._project(ctx, h)
+    def forward_out_projected(self, ctx, call, proj, out) -> None:
+        self._run(ctx, call, None, out, False, projected=proj)
+
+    def _run(self, ctx, call, h, target, add: bool, projected=None) -> None:
+        y = projected if projected is not None else self._project(ctx, h)
         if self.rot:
             ops.rotate_halves_rows(y, (self.offsets["q"], self.offsets["k"]), self.heads, self.dim, self.rot, self.cos, self.sin,
                                    ctx.positions, ctx.rows)

@@ -16,12 +16,15 @@ import torch
 
 from ..csrc import ops
 from .base import MIXERS, CacheSpec, Mixer, PartSpec, StateSpec, TensorSpec, lookup, register_mixer
+from .linear import Linear
 
 
 @register_mixer("side_by_side")
 class SideBySide(Mixer):
     """params: width, eps, branches: a list of (name, PartSpec of a mixer); a branch's tensors are its own behind
     ``<name>.``, and ``<name>.out`` [width] is the weight of the norm behind it."""
+
+    SHARED_MAX_ROWS = 64       # steps of up to this many rows run the branches' first products as one
 
     def __init__(self, params, runtime):
         super().__init__(params, runtime)
@@ -69,8 +72,24 @@ class SideBySide(Mixer):
         for name, b in zip(self.names, self.branches):
             b.bind({t: tensors[f"{name}.{t}"] for t in b.tensors()})
         self.out_weights = [tensors[f"{name}.out"].to(self.rt.device).float().contiguous() for name in self.names]
+        # Branches whose whole reading of the input is one product each share one product: the matrices stacked (the
+        # branches keep blocks of the stacked matrix, no copies), the branches read their columns of it.  A product's
+        # column does not depend on the columns beside it, so these are the bits of a product each.
+        self.shared_projection: Optional[Linear] = None
+        self.shared_columns: List[Tuple[int, int]] = []
+        firsts = [b.input_projection() for b in self.branches]
+        if len(self.branches) > 1 and all(p is not None for p in firsts) and len({p.weight.dtype for p in firsts}) == 1 \
+                and len({p.mfma for p in firsts}) == 1:
+            self.shared_projection = Linear(torch.cat([p.weight for p in firsts], dim=0), self.rt)
+            at = 0
+            for b, p in zip(self.branches, firsts):
+                n = p.out_features
+                b.adopt_input_projection(self.shared_projection.weight[at:at + n])
+                self.shared_columns.append((at, n))
+                at += n
 
     def weight_bytes(self) -> int:
+        # (a branch counts its block of the shared matrix as its own projection)
         return sum(b.weight_bytes() for b in self.branches) + 4 * self.width * len(self.branches)
 
     def cache_spec(self) -> Optional[CacheSpec]:
@@ -115,9 +134,19 @@ class SideBySide(Mixer):
 
     def _branch_outputs(self, ctx, call, h):
         ys = []
+        projected = None
+        # (steps of few rows, where a launch costs more than its arithmetic; a prompt portion's two products run faster apart
+        # than one of their joint, odd number of columns: 2,048 rows of 2,576 + 6,144 columns took 0.14 ms longer as one)
+        if self.shared_projection is not None and ctx.rows <= self.SHARED_MAX_ROWS:
+            projected = ctx.ws.buffer("side_by_side_projected", self.shared_projection.out_features, torch.float32)
+            self.shared_projection.store(ctx.ws, h, projected, ctx.rows)
         for i, (b, sub) in enumerate(zip(self.branches, self._branch_calls(ctx, call))):
             y = ctx.ws.buffer(f"side_by_side_{i}", self.width, torch.float32)
-            b.forward_out(ctx, sub, h, y)
+            if projected is not None:
+                at, n = self.shared_columns[i]
+                b.forward_out_projected(ctx, sub, projected[:, at:at + n], y)
+            else:
+                b.forward_out(ctx, sub, h, y)
             ys.append(y)
         return ys
 
