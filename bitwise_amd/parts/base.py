@@ -259,6 +259,12 @@ class Mixer(Part):
         norm and ``forward`` one after the other.  The result must be the same bits."""
         return False
 
+    def forward_between_norms(self, ctx, call, x, norm, norm_behind) -> bool:
+        """Optional: x += norm_behind(mixer(norm(x))) with both norms riding in the mixer's own launches (the one in front in
+        its first product, the one behind in its last kernel).  Return False (and do nothing) if this step cannot; the
+        block then runs the norm in front and goes on as without this.  The result must be the same bits."""
+        return False
+
     def input_projection(self):
         """Optional: the ``Linear`` whose product of the mixer's input (32-bit sums) is all the mixer reads of its input, or
         None.  A mixer that names one also takes ``adopt_input_projection(weight)`` (the same rows, now a block of a larger

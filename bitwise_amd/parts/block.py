@@ -140,11 +140,13 @@ class SandwichBlock(Block):
         return self.mixer_norm.state_spec()
 
     def forward(self, ctx, call, x) -> None:
-        if call.block_state is not None:
+        if call.block_state is None and self.mixer.forward_between_norms(ctx, call, x, self.mixer_norm, self.mixer_post_norm):
+            h = None
+        elif call.block_state is not None:
             h = self.mixer_norm.forward(ctx, x, state=call.block_state)
         else:
             h = self.mixer_norm.forward(ctx, x)
-        if not self.mixer.forward_add_normed(ctx, call, h, self.mixer_post_norm, x):
+        if h is not None and not self.mixer.forward_add_normed(ctx, call, h, self.mixer_post_norm, x):
             y = ctx.ws.buffer("sublayer_out", x.shape[1], torch.float32)
             self.mixer.forward_out(ctx, call, h, y)
             self.mixer_post_norm.add_normed(ctx, y, x)

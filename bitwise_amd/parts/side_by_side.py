@@ -132,12 +132,11 @@ class SideBySide(Mixer):
             return calls
         return ctx.memo(("side_by_side_calls", id(self), call.index), make)
 
-    def _branch_outputs(self, ctx, call, h):
+    def _branch_outputs(self, ctx, call, h, projected=None):
         ys = []
-        projected = None
         # (steps of few rows, where a launch costs more than its arithmetic; a prompt portion's two products run faster apart
         # than one of their joint, odd number of columns: 2,048 rows of 2,576 + 6,144 columns took 0.14 ms longer as one)
-        if self.shared_projection is not None and ctx.rows <= self.SHARED_MAX_ROWS:
+        if projected is None and self.shared_projection is not None and ctx.rows <= self.SHARED_MAX_ROWS:
             projected = ctx.ws.buffer("side_by_side_projected", self.shared_projection.out_features, torch.float32)
             self.shared_projection.store(ctx.ws, h, projected, ctx.rows)
         for i, (b, sub) in enumerate(zip(self.branches, self._branch_calls(ctx, call))):
@@ -153,15 +152,34 @@ class SideBySide(Mixer):
     def forward_out(self, ctx, call, h, out) -> None:
         ops.norm_mean(self._branch_outputs(ctx, call, h), self.out_weights, out, ctx.rows, self.eps)
 
-    def forward_add_normed(self, ctx, call, h, norm, x) -> bool:
-        """The norm behind the mixer rides in the launch that norms and averages the branches (the same bits)."""
+    def _can_ride(self, norm) -> bool:
         from .norm import RMSNorm
-        if type(norm) is not RMSNorm or self.width > ops.NORM_MEAN_ADD_MAX_WIDTH:
-            return False
+        return type(norm) is RMSNorm and self.width <= ops.NORM_MEAN_ADD_MAX_WIDTH
+
+    def _mean_add(self, ctx, ys, norm, x) -> None:
         w32 = self._post_weights.get(id(norm))
         if w32 is None:
             w32 = self._post_weights[id(norm)] = norm.weight.float().contiguous()       # (widening is exact)
-        ops.norm_mean_add(self._branch_outputs(ctx, call, h), self.out_weights, self.eps, w32, norm.eps, norm.scale, x, ctx.rows)
+        ops.norm_mean_add(ys, self.out_weights, self.eps, w32, norm.eps, norm.scale, x, ctx.rows)
+
+    def forward_add_normed(self, ctx, call, h, norm, x) -> bool:
+        """The norm behind the mixer rides in the launch that norms and averages the branches (the same bits)."""
+        if not self._can_ride(norm):
+            return False
+        self._mean_add(ctx, self._branch_outputs(ctx, call, h), norm, x)
+        return True
+
+    def forward_between_norms(self, ctx, call, x, norm, norm_behind) -> bool:
+        """Decode steps of few rows: the norm in front rides in the branches' one product (the bits of norm, then
+        product), the norm behind in the launch that averages the branches."""
+        from .norm import RMSNorm
+        sp = self.shared_projection
+        if not (sp is not None and self.rt.bf16 and sp.mfma and type(norm) is RMSNorm and self._can_ride(norm_behind)
+                and ctx.rows <= self.SHARED_MAX_ROWS and ops.can_fuse_norm(ctx.rows, sp.weight, x)):
+            return False
+        projected = ctx.ws.buffer("side_by_side_projected", sp.out_features, torch.float32)
+        ops.norm_gemm_bf16(x, norm.weight, norm.eps, sp.weight, projected, ctx.rows, ops.EPI_F32)
+        self._mean_add(ctx, self._branch_outputs(ctx, call, None, projected), norm_behind, x)
         return True
 
     def forward(self, ctx, call, h, residual) -> None:
