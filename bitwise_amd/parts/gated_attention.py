@@ -51,10 +51,12 @@ def max_seq_rows(ctx) -> int:
 
 @register_mixer("gated_attention")
 class GatedAttention(Mixer):
-    """params: width, heads, kv_heads, dim, vdim, scale, eps, conv (taps), qk_norm, sink, gate, shared_kv, window,
-    position (PartSpec of a position encoding with the layout "pairs").
-    tensors: q, k, v [heads*dim | kv_heads*dim | kv_heads*vdim, width]; q.conv, k.conv, v.conv [channels, taps];
-    g [heads*vdim, width]; o [width, heads*vdim]."""
+    """params: width, heads, kv_heads, dim, vdim, scale, eps, conv (taps), qk_norm, sink (None, a number or "learned"), gate
+    (False, True or "head"), values ("own" or "keys"), shared_kv, window, softcap, chunk, v_mix, position (PartSpec of a
+    position encoding with the layout "pairs" or "halves").
+    tensors: q, k, v [heads*dim | kv_heads*dim | kv_heads*vdim, width] (no v where the values are the keys); q.conv, k.conv,
+    v.conv [channels, taps]; g [heads*vdim, width] (a gate a head: [heads, width]); sink [heads] if learned;
+    o [width, heads*vdim]."""
 
     graph_safe = True
     launches_through_ops = True
